@@ -1,0 +1,166 @@
+"""Benchmark of the paged KV-cache hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one paged decode attention (split kernel + merge kernel) over the Qwen3-8B-shaped
+decode batch (32 query heads, 8 KV heads, head_dim 128, block 256, batch 64, context lengths
+uniform in [512, 4096], block tables shuffled over a pool 1.2x the need).  Inputs are resident
+in HBM before the clock starts.  Successive steps walk over several independent copies of the
+cache (as successive layers of a model do) so that the 256 MB Infinity Cache cannot serve the
+reads.  Prints one JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+HBM_PEAK_GBS = 8000.0
+
+
+def gpu_time_ms(fn, iters, warmup):
+    """Average milliseconds per call of ``fn`` over ``iters`` calls, HIP events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def cpu_baseline(sample_seqs=16, min_seconds=10.0):
+    """The CPU restatement of the same path (gather + SDPA, oracle/torch_path.py) on the host cores,
+    over a bounded sample of the same workload: the first ``sample_seqs`` sequences of the batch."""
+    from infer_amd import workloads
+    from oracle import torch_path
+    lengths = workloads.cfg2_lengths()[:sample_seqs]
+    wl = workloads.make_decode_workload("cfg2-sample", lengths, 32, 8, seed=0, q_scale=128 ** -0.5)
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    torch_path.paged_decode_torch(wl.q, wl.k_cache, wl.v_cache, wl.block_table, wl.context_lens, wl.scale)
+    times = []
+    t_end = time.perf_counter() + min_seconds
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 50):
+        t0 = time.perf_counter()
+        torch_path.paged_decode_torch(wl.q, wl.k_cache, wl.v_cache, wl.block_table, wl.context_lens, wl.scale)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {
+        "value": round(wl.decode_bytes / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+        "sample": f"first {sample_seqs} of the 64 sequences ({sum(lengths)} tokens, "
+                  f"{wl.decode_bytes / 1e6:.1f} MB algorithmic), median of {len(times)} runs, "
+                  f"torch {torch.get_num_threads()} threads",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--copies", type=int, default=4, help="independent cache copies walked round-robin")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--splits", type=int, default=0, help="KV-split workgroups (0 = library default)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this path needs no collective and every box here has one GPU; "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU: the HIP kernels are the only implementation of the path", file=sys.stderr)
+        sys.exit(2)
+
+    from infer_amd import ops, workloads
+    dev = torch.device("cuda:0")
+    if args.splits:
+        ops.set_split_workgroups(args.splits)
+    wl = workloads.cfg2(device=dev)
+    b, hq, hkv, d = len(wl.lengths), wl.num_q_heads, wl.num_kv_heads, wl.head_dim
+    k_copies = [wl.k_cache] + [torch.randn_like(wl.k_cache) for _ in range(args.copies - 1)]
+    v_copies = [wl.v_cache] + [torch.randn_like(wl.v_cache) for _ in range(args.copies - 1)]
+    out = torch.empty((b, hq, d), dtype=torch.bfloat16, device=dev)
+    ws = ops.decode_workspace(dev, b, hq, hkv, d)
+    it = [0]
+
+    def step():
+        i = it[0] % args.copies
+        it[0] += 1
+        ops.paged_attn_decode(wl.q, k_copies[i], v_copies[i], wl.block_table, wl.context_lens, wl.scale, out, ws)
+
+    def split_only():
+        i = it[0] % args.copies
+        it[0] += 1
+        ops.paged_attn_decode_split(wl.q, k_copies[i], v_copies[i], wl.block_table, wl.context_lens, wl.scale, ws)
+
+    # whole op, exactly K steps
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = gpu_time_ms(step, args.steps, 0)
+    ms_per_step = max(ms_per_step, 1e-6)
+    nbytes = wl.decode_bytes
+    value = nbytes / (ms_per_step * 1e-3) / 1e9
+
+    # dominant kernel alone (the KV-streaming split kernel)
+    split_ms = gpu_time_ms(split_only, args.steps, 5)
+    achieved = nbytes / (split_ms * 1e-3) / 1e9
+
+    # KV append: decode-sized (64 rows, latency bound) and prefill-sized (cfg3)
+    ap_small_ms = gpu_time_ms(lambda: ops.store_kvcache(wl.k_new, wl.v_new, wl.k_cache, wl.v_cache, wl.slot_mapping),
+                              args.steps, 5)
+    p3 = workloads.cfg3(device=dev)
+    reps = 24   # distinct source/destination buffers walked round-robin (24 x ~100 MB > Infinity Cache)
+    srcs = [(torch.randn_like(p3.k_new), torch.randn_like(p3.v_new)) for _ in range(reps)]
+    dsts = [(torch.empty_like(p3.k_cache), torch.empty_like(p3.v_cache)) for _ in range(reps)]
+    jt = [0]
+
+    def append_step():
+        j = jt[0] % reps
+        jt[0] += 1
+        ops.store_kvcache(srcs[j][0], srcs[j][1], dsts[j][0], dsts[j][1], p3.slot_mapping)
+
+    ap_ms = gpu_time_ms(append_step, max(args.steps, 48), reps)
+    append_gbs = p3.append_bytes / (ap_ms * 1e-3) / 1e9
+
+    line = {
+        "metric": "paged decode attn HBM GB/s (% of 8 TB/s peak), Qwen3-8B shapes bs=64",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "cfg2: paged decode attention, Hq=32 Hkv=8 D=128 block=256 batch=64 "
+                               "ctx~U[512,4096] (seed 0), tables shuffled over a 1.2x pool",
+                   "tokens": sum(wl.lengths), "algorithmic_bytes": nbytes, "cache_copies": args.copies,
+                   "split_workgroups": args.splits or "default"},
+        "pct_of_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "wall_ms_per_step": round(wall_ms, 5),
+        "roofline": {"bound": "hbm", "kernel": "paged_decode_split_kernel", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": None, "avg_kernel_ms": round(split_ms, 5)},
+        "append": {"decode_rows": b, "decode_us": round(ap_small_ms * 1e3, 2),
+                   "prefill_rows": int(p3.slot_mapping.numel()), "prefill_bytes": p3.append_bytes,
+                   "prefill_us": round(ap_ms * 1e3, 2), "prefill_GBps": round(append_gbs, 1),
+                   "prefill_frac_of_peak": round(append_gbs / HBM_PEAK_GBS, 4)},
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,135 @@
+/* infer_kv.h - C ABI of libinfer_kv.so: the paged KV-cache hot path on MI355X (gfx950).
+ *
+ * Three pieces, one library:
+ *   1. KV append         - slot_mapping-driven scatter of new K/V rows into the paged caches.
+ *   2. Paged decode attn - block_table-gathered GQA attention of one query token per sequence.
+ *   3. Block pool        - host-side allocator of cache blocks with a prefix cache.
+ *
+ * Conventions for every device entry point:
+ *   - all pointers are device pointers unless the name says "host"; they are borrowed for the
+ *     duration of the call on `stream` (a hipStream_t passed as void*; NULL = default stream);
+ *   - the call only enqueues work: it never synchronises, never allocates, never frees, and
+ *     never throws; it is safe to record into a HIP graph;
+ *   - return value: 0 on success, a negative INFER_KV_E* code for a rejected argument, or a
+ *     positive hipError_t reported by the launch;
+ *   - element type is bfloat16 (the only type the reference instantiates: src/kvcache.cc:305),
+ *     strides are in ELEMENTS, metadata is int32.
+ *
+ * The reference has no FFI of its own for this path: the append is a Triton kernel and the
+ * attention is the pip package flash_attn, both called from Python.  Each declaration below
+ * cites the reference call it replaces (paths into the reference tree).
+ */
+#ifndef INFER_KV_H
+#define INFER_KV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define INFER_KV_OK            0
+#define INFER_KV_EINVAL       -1   /* null pointer, non-positive size, unsupported shape        */
+#define INFER_KV_EALIGN       -2   /* pointer or stride not aligned for the vector path         */
+#define INFER_KV_EWORKSPACE   -3   /* workspace too small                                       */
+#define INFER_KV_EUNSUPPORTED -4   /* head_dim / group size / block size outside what is built  */
+
+/* Library version, "major.minor". */
+const char* infer_kv_version(void);
+
+/* Human-readable text for a code returned by any entry point (negative codes: this library;
+ * positive: hipGetErrorString). */
+const char* infer_kv_strerror(int code);
+
+/* ------------------------------------------------------------------ 1. KV append
+ * Replaces store_kvcache / store_kvcache_kernel (infer/ops/attention.py:16-45), called from
+ * Attention.forward_offical_fa_impl (infer/ops/attention.py:108-109).
+ *
+ * For every row i in [0, n_rows): slot = slot_mapping[i]; if 0 <= slot < num_slots then
+ *   k_cache[slot * dkv .. +dkv) = key[i * key_stride0 .. +dkv)   (same for value -> v_cache).
+ * Rows whose slot is negative (padding) or >= num_slots are skipped; the reference has no such
+ * guard (a -1 slot writes out of bounds there).  dkv = num_kv_heads * head_dim; the caches are
+ * [num_slots, dkv] row-major (the reference asserts k_cache.stride(1) == dkv).  key/value rows
+ * may be strided views of a fused qkv projection (row stride != dkv) but each row is contiguous.
+ * Duplicate slots in one call race (last writer unspecified), as in the reference.
+ * Requires dkv % 8 == 0 and 16-byte aligned rows (pointers and strides), else INFER_KV_EALIGN.
+ */
+int infer_kv_append_bf16(const void* key, int64_t key_stride0,
+                         const void* value, int64_t value_stride0,
+                         void* k_cache, void* v_cache,
+                         const int32_t* slot_mapping,
+                         int64_t n_rows, int64_t dkv, int64_t num_slots,
+                         void* stream);
+
+/* ------------------------------------------------------------------ 2. paged decode attention
+ * Replaces flash_attn_with_kvcache(q[B,1,Hq,D], k_cache, v_cache, cache_seqlens=context_lens,
+ * block_table=block_tables, softmax_scale=scale, causal=True) at infer/ops/attention.py:118-120,
+ * and is the body the stub src/operators/flashattn/flashattn_decode.cu:11-13 never got.
+ *
+ *   out[b, h, :] = softmax_t( scale * q[b, h, :] . K_b[t, h / G, :] ) V_b[t, h / G, :],
+ *   t in [0, context_lens[b]),  G = num_q_heads / num_kv_heads,
+ *   K_b[t] = k_cache[block_table[b, t / block_size], t % block_size]   (same for V).
+ *
+ * Rows with context_lens[b] <= 0 (graph padding) write zeros.  Table entries past
+ * ceil(len / block_size) are never read; entries that are read are clamped into
+ * [0, num_blocks) so a corrupt table cannot fault the GPU.
+ *
+ * Layouts (strides in elements): q [B, Hq, D] with row stride q_stride0, heads contiguous;
+ * out likewise with out_stride0; caches [num_blocks, block_size, Hkv, D] with block stride
+ * cache_block_stride and token stride cache_token_stride (heads contiguous, D innermost);
+ * block_table [B, *] with row stride bt_stride0; context_lens [B].
+ *
+ * The work is split across workgroups in equal shares of KV tokens regardless of sequence
+ * boundaries; partial (max, sum, accumulator) results go to `workspace` and are merged by a
+ * second small kernel.  Size the workspace with infer_paged_decode_workspace_bytes() for the
+ * largest batch that will be passed; its contents need no initialisation.
+ *
+ * Built for head_dim == 128, 1 <= G <= 16, block_size % 32 == 0 (the reference requires a
+ * multiple of 256: infer/config.py:21), num_kv_heads <= 8 or a multiple of 8.
+ */
+size_t infer_paged_decode_workspace_bytes(int64_t max_batch, int64_t num_q_heads,
+                                          int64_t num_kv_heads, int64_t head_dim);
+
+int infer_paged_decode_bf16(const void* q, int64_t q_stride0,
+                            const void* k_cache, const void* v_cache,
+                            int64_t cache_block_stride, int64_t cache_token_stride,
+                            void* out, int64_t out_stride0,
+                            const int32_t* block_table, int64_t bt_stride0,
+                            const int32_t* context_lens,
+                            int64_t batch, int64_t num_q_heads, int64_t num_kv_heads,
+                            int64_t head_dim, int64_t block_size, int64_t num_blocks,
+                            float scale,
+                            void* workspace, size_t workspace_bytes,
+                            void* stream);
+
+/* The two phases of infer_paged_decode_bf16 on their own (same arguments): `split` streams the
+ * KV cache and leaves partial results in the workspace, `merge` combines them into `out`.
+ * Calling split then merge on one stream is exactly infer_paged_decode_bf16.  They exist so a
+ * profiler or a benchmark can time the bandwidth-bound phase alone. */
+int infer_paged_decode_split_bf16(const void* q, int64_t q_stride0,
+                                  const void* k_cache, const void* v_cache,
+                                  int64_t cache_block_stride, int64_t cache_token_stride,
+                                  const int32_t* block_table, int64_t bt_stride0,
+                                  const int32_t* context_lens,
+                                  int64_t batch, int64_t num_q_heads, int64_t num_kv_heads,
+                                  int64_t head_dim, int64_t block_size, int64_t num_blocks,
+                                  float scale,
+                                  void* workspace, size_t workspace_bytes,
+                                  void* stream);
+
+int infer_paged_decode_merge_bf16(void* out, int64_t out_stride0,
+                                  const int32_t* context_lens,
+                                  int64_t batch, int64_t num_q_heads, int64_t num_kv_heads,
+                                  int64_t head_dim,
+                                  const void* workspace, size_t workspace_bytes,
+                                  void* stream);
+
+/* Tuning knob: number of workgroups along the KV-split axis used by the decode kernels
+ * (0 = choose from the device's CU count).  Process-wide; returns the previous value. */
+int infer_paged_decode_set_split_workgroups(int workgroups);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* INFER_KV_H */

@@ -1,0 +1,58 @@
+"""ctypes binding of ``libinfer_kv.so`` (see ``include/infer_kv.h`` for the contract).
+
+The library is built in-tree by ``infer_amd/csrc/Makefile``.  There is no fallback: if the
+library is missing, loading raises ``ImportError`` and every op that needs it fails loudly.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libinfer_kv.so")
+
+_lock = threading.Lock()
+_lib = None
+
+_c = ctypes
+_i64, _i32, _f32, _vp, _sz = _c.c_int64, _c.c_int32, _c.c_float, _c.c_void_p, _c.c_size_t
+
+# name -> (restype, argtypes); mirrors include/infer_kv.h declaration by declaration
+SIGNATURES = {
+    "infer_kv_version": (_c.c_char_p, []),
+    "infer_kv_strerror": (_c.c_char_p, [_c.c_int]),
+    "infer_kv_append_bf16": (_c.c_int, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "infer_paged_decode_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64]),
+    "infer_paged_decode_bf16": (_c.c_int, [_vp, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _i64, _vp,
+                                           _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp, _sz, _vp]),
+    "infer_paged_decode_split_bf16": (_c.c_int, [_vp, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _vp,
+                                                 _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp, _sz, _vp]),
+    "infer_paged_decode_merge_bf16": (_c.c_int, [_vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _sz, _vp]),
+    "infer_paged_decode_set_split_workgroups": (_c.c_int, [_c.c_int]),
+}
+
+
+def load():
+    """Load the shared library once and attach argument types.  Raises ImportError if absent."""
+    global _lib
+    with _lock:
+        if _lib is None:
+            if not os.path.exists(LIB_PATH):
+                raise ImportError(
+                    f"{LIB_PATH} is not built; run `make -C infer_amd/csrc` (or __graft_entry__.build())")
+            lib = ctypes.CDLL(LIB_PATH)
+            for name, (res, args) in SIGNATURES.items():
+                fn = getattr(lib, name)
+                fn.restype = res
+                fn.argtypes = args
+            _lib = lib
+    return _lib
+
+
+def check(code: int, what: str) -> None:
+    """Turn a non-zero return code into RuntimeError (the reference's ops raise RuntimeError through
+    TORCH_CHECK / std::runtime_error, e.g. src/operators/flashattn/flashattn.cu:272)."""
+    if code != 0:
+        msg = load().infer_kv_strerror(code).decode()
+        raise RuntimeError(f"{what} failed: {msg} (code {code})")

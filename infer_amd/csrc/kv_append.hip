@@ -1,0 +1,103 @@
+// KV append for gfx950 (MI355X): scatter new K/V rows into the paged caches, keyed by slot.
+//
+// Replaces store_kvcache_kernel / store_kvcache (infer/ops/attention.py:16-45 of the
+// reference): cache.flat[slot * dkv .. +dkv) = row.  Unlike the reference, rows whose slot is
+// negative (padding) or past the end of the cache are skipped instead of written out of bounds.
+//
+// One wavefront copies one token: its K row and its V row, 16 bytes per lane per access, all
+// loads of a row pair issued before the first store.  Pure byte movement, so the result is
+// bit-exact by construction; the kernel is bound by HBM bandwidth (rows in, rows out).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/infer_kv.h"
+
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWavesPerBlock = 4;
+
+// CHUNKS = 16-byte chunks per lane and row when the row is exactly 64 * CHUNKS chunks wide;
+// CHUNKS == 0 is the generic strided loop.
+template <int CHUNKS>
+__global__ void __launch_bounds__(64 * kWavesPerBlock)
+kv_append_kernel(const u32x4* __restrict__ key, int64_t key_stride_v, const u32x4* __restrict__ value,
+                 int64_t value_stride_v, u32x4* __restrict__ k_cache, u32x4* __restrict__ v_cache,
+                 const int32_t* __restrict__ slot_mapping, int64_t n_rows, int row_chunks, int64_t num_slots) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    if (row >= n_rows) return;
+    const int64_t slot = __builtin_amdgcn_readfirstlane(slot_mapping[row]);
+    if (slot < 0 || slot >= num_slots) return;
+    const u32x4* ks = key + row * key_stride_v;
+    const u32x4* vs = value + row * value_stride_v;
+    u32x4* kd = k_cache + slot * row_chunks;
+    u32x4* vd = v_cache + slot * row_chunks;
+    if (CHUNKS > 0) {
+        u32x4 kr[CHUNKS > 0 ? CHUNKS : 1], vr[CHUNKS > 0 ? CHUNKS : 1];
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c) kr[c] = __builtin_nontemporal_load(ks + lane + 64 * c);
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c) vr[c] = __builtin_nontemporal_load(vs + lane + 64 * c);
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c) kd[lane + 64 * c] = kr[c];
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c) vd[lane + 64 * c] = vr[c];
+    } else {
+        for (int c = lane; c < row_chunks; c += 64) {
+            u32x4 kr = ks[c];
+            u32x4 vr = vs[c];
+            kd[c] = kr;
+            vd[c] = vr;
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int infer_kv_append_bf16(const void* key, int64_t key_stride0, const void* value, int64_t value_stride0,
+                         void* k_cache, void* v_cache, const int32_t* slot_mapping, int64_t n_rows, int64_t dkv,
+                         int64_t num_slots, void* stream) {
+    if (n_rows == 0) return INFER_KV_OK;
+    if (!key || !value || !k_cache || !v_cache || !slot_mapping) return INFER_KV_EINVAL;
+    if (n_rows < 0 || dkv <= 0 || num_slots <= 0) return INFER_KV_EINVAL;
+    if (key_stride0 < dkv || value_stride0 < dkv) return INFER_KV_EINVAL;
+    if (dkv % 8 != 0 || key_stride0 % 8 != 0 || value_stride0 % 8 != 0) return INFER_KV_EALIGN;
+    if (((uintptr_t)key | (uintptr_t)value | (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) return INFER_KV_EALIGN;
+    if ((n_rows + kWavesPerBlock - 1) / kWavesPerBlock > 0x7fffffffLL) return INFER_KV_EINVAL;
+    const int row_chunks = (int)(dkv / 8);
+    dim3 grid((unsigned)((n_rows + kWavesPerBlock - 1) / kWavesPerBlock), 1, 1), block(64 * kWavesPerBlock, 1, 1);
+    hipStream_t st = (hipStream_t)stream;
+#define INFER_KV_LAUNCH_APPEND(C)                                                                          \
+    hipLaunchKernelGGL(kv_append_kernel<C>, grid, block, 0, st, (const u32x4*)key, key_stride0 / 8,        \
+                       (const u32x4*)value, value_stride0 / 8, (u32x4*)k_cache, (u32x4*)v_cache,           \
+                       slot_mapping, n_rows, row_chunks, num_slots)
+    switch (row_chunks) {
+        case 64: INFER_KV_LAUNCH_APPEND(1); break;
+        case 128: INFER_KV_LAUNCH_APPEND(2); break;
+        case 256: INFER_KV_LAUNCH_APPEND(4); break;
+        default: INFER_KV_LAUNCH_APPEND(0); break;
+    }
+#undef INFER_KV_LAUNCH_APPEND
+    return (int)hipGetLastError();
+}
+
+const char* infer_kv_version(void) { return "0.1"; }
+
+const char* infer_kv_strerror(int code) {
+    switch (code) {
+        case INFER_KV_OK: return "ok";
+        case INFER_KV_EINVAL: return "invalid argument (null pointer, non-positive size or inconsistent stride)";
+        case INFER_KV_EALIGN: return "pointer or stride not 16-byte aligned";
+        case INFER_KV_EWORKSPACE: return "workspace too small";
+        case INFER_KV_EUNSUPPORTED: return "shape not built (head_dim must be 128, group size <= 16, block_size % 32 == 0)";
+        default: break;
+    }
+    if (code > 0) return hipGetErrorString((hipError_t)code);
+    return "unknown error";
+}
+
+}  // extern "C"

@@ -1,0 +1,526 @@
+// Paged decode attention for gfx950 (MI355X): block_table-gathered GQA attention of one query
+// token per sequence, flash-decoding style (split KV + merge), bf16 in / fp32 accumulate.
+//
+// Replaces flash_attn_with_kvcache(...) at infer/ops/attention.py:118-120 of the reference
+// (the reference's own decode kernel, src/operators/flashattn/flashattn_decode.cu, is an empty
+// stub).  The merge rule for partial (max, sum) pairs is the same algebra as the reference's
+// softmax reduction (src/operators/softmax/softmax.cu:5-16).
+//
+// Work decomposition
+//   A "step" is 32 consecutive tokens of one sequence (never straddles a cache block because
+//   block_size % 32 == 0).  All steps of all sequences are laid end to end and cut into
+//   gridDim.x equal spans; workgroup x streams span x for up to 8 KV heads, one wavefront per
+//   KV head, so a workgroup reads whole 2 KiB token rows while each wavefront runs its own
+//   private pipeline (no workgroup barrier anywhere).  A span may cover the tail of one
+//   sequence and the head of the next: each (sequence, span) piece is a "segment" and leaves a
+//   partial result; the merge kernel folds the segments of a sequence together.
+//
+// Per step and wavefront (KV head h, G = Hq/Hkv query heads):
+//   S^T[token, head] = K[token, :] . Q^T        2 tiles x 4 v_mfma_f32_16x16x32_bf16
+//   online softmax in the MFMA accumulator layout (lane = head, 8 tokens per lane)
+//   O^T[d, head]    += V^T[d, token] . P^T      8 v_mfma_f32_16x16x32_bf16
+//   K fragments are loaded straight from global memory in MFMA operand layout (16 B per lane);
+//   V rows are loaded coalesced (256 B per token), staged in a wave-private LDS tile and read
+//   back transposed.  The accumulator layout of S^T is exactly the B-operand layout of the
+//   second product, so P never moves between lanes.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "decode_layout.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kD = 128;            // head_dim
+constexpr int kStep = 32;          // tokens per step
+constexpr int kLdsRow = 288;       // bytes per staged V row: 256 + 32 so 4 consecutive rows hit disjoint banks
+constexpr int kLdsWave = kStep * kLdsRow;
+constexpr int kMinSpan = 4;        // steps; keeps partial-result traffic small on tiny problems
+
+struct DecodeArgs {
+    const uint16_t* q;
+    int64_t q_stride0;
+    const uint16_t* k;
+    const uint16_t* v;
+    int64_t blk_stride;
+    int64_t tok_stride;
+    const int32_t* bt;
+    int64_t bt_stride0;
+    const int32_t* ctx;
+    int batch;
+    int group;          // query heads per KV head
+    int num_kv_heads;
+    int block_size;
+    int num_blocks;
+    float scale_log2;   // softmax scale * log2(e)
+    int32_t* header;
+    int32_t* seg_first;
+    int32_t* seg_last;
+    float* ml;          // [slots][group][2]
+    float* po;          // [slots][group][128]
+    int slots_per_head; // gridDim.x + batch
+};
+
+__device__ __forceinline__ bf16x8 as_bf16x8(u32x4 x) { return __builtin_bit_cast(bf16x8, x); }
+
+__device__ __forceinline__ u32x4 load16(const uint16_t* p) {
+    return *reinterpret_cast<const u32x4*>(p);
+}
+
+__device__ __forceinline__ int steps_of(int len) { return len > 0 ? (len + kStep - 1) / kStep : 0; }
+
+__device__ __forceinline__ int wave_sum(int x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
+    return x;
+}
+
+__device__ __forceinline__ int wave_inclusive_scan(int x, int lane) {
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        int y = __shfl_up(x, o);
+        if (lane >= o) x += y;
+    }
+    return x;
+}
+
+// Keeps the compiler from moving LDS traffic across this point.  The LDS queue of one
+// wavefront is processed in order, so within a wavefront a compiler barrier is all the
+// write -> read -> write sequence on the private tile needs.
+__device__ __forceinline__ void lds_order() { __asm__ volatile("" ::: "memory"); }
+
+// One (sequence, span) piece: steps [s_lo, s_hi) of sequence b for KV head h.
+__device__ __forceinline__ void run_segment(const DecodeArgs& a, unsigned char* lds, int b, int len,
+                                            int s_lo, int s_hi, int h, int w, int lane) {
+    const int g = lane >> 4;   // lane group: the k-slice of MFMA operands, the row-quad of results
+    const int n = lane & 15;   // operand row / result column
+    const int G = a.group;
+
+    // Q as the B operand of S^T = K Q^T: lane (g, n) holds Q[head n][32 j + 8 g .. +8].
+    bf16x8 qreg[4];
+    {
+        u32x4 z = {0u, 0u, 0u, 0u};
+        const uint16_t* qp = a.q + (int64_t)b * a.q_stride0 + (int64_t)(h * G + (n < G ? n : 0)) * kD + 8 * g;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) qreg[j] = as_bf16x8(n < G ? load16(qp + 32 * j) : z);
+    }
+
+    f32x4 acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY;
+    float l_run = 0.f;
+
+    // Block ids of the segment: lane i keeps the table entry of block (tbl_base + i), so the
+    // per-step lookup is a register read instead of a dependent memory load.
+    const int32_t* btrow = a.bt + (int64_t)b * a.bt_stride0;
+    const int steps_per_blk = a.block_size / kStep;
+    const int blk_last = (s_hi - 1) / steps_per_blk;
+    int tbl_base = s_lo / steps_per_blk;
+    int tblv = (tbl_base + lane <= blk_last) ? btrow[tbl_base + lane] : 0;
+    int nxt_bi = tbl_base;                       // block index (within the sequence) of the next step to load
+    int nxt_in = s_lo - tbl_base * steps_per_blk; // its step index inside that block
+
+    // Row r of a K tile holds token 4 (r % 4) + r / 4 of the tile, so that result element
+    // (tile t, quad element e) of lane group g is token 4 (4 t + e) + g of the step.
+    const uint32_t k_lane = (uint32_t)((4 * (n & 3) + (n >> 2)) * a.tok_stride + 8 * g);
+    const uint32_t v_lane = (uint32_t)(g * a.tok_stride + 8 * n);
+    const uint32_t tile_off = (uint32_t)(16 * a.tok_stride);
+    const uint32_t quad_off = (uint32_t)(4 * a.tok_stride);
+
+    u32x4 kreg[2][4];
+    u32x4 vreg[8];
+
+    // Issues the 16 loads of the next step in line and advances the (block, step-in-block) cursor.
+    auto issue_loads = [&]() {
+        if (nxt_bi - tbl_base >= 64) {   // only for segments longer than 64 blocks
+            tbl_base = nxt_bi;
+            tblv = (tbl_base + lane <= blk_last) ? btrow[tbl_base + lane] : 0;
+        }
+        int blk = __builtin_amdgcn_readlane(tblv, nxt_bi - tbl_base);
+        blk = blk < 0 ? 0 : (blk >= a.num_blocks ? a.num_blocks - 1 : blk);
+        const int64_t base = (int64_t)blk * a.blk_stride + (int64_t)(nxt_in * kStep) * a.tok_stride + (int64_t)h * kD;
+        const uint16_t* kb = a.k + base;
+        const uint16_t* vb = a.v + base;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) kreg[t][j] = load16(kb + (t * tile_off + k_lane) + 32 * j);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) vreg[i] = load16(vb + (i * quad_off + v_lane));
+        if (++nxt_in == steps_per_blk) {
+            nxt_in = 0;
+            ++nxt_bi;
+        }
+    };
+
+    issue_loads();
+
+    for (int s = s_lo; s < s_hi; ++s) {
+        // ---- S^T = K Q^T
+        f32x4 sc[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            sc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kreg[t][j]), qreg[j], sc[t], 0, 0, 0);
+        }
+
+        // ---- stage V (rows past the end of the sequence are zeroed: their P is 0 and 0 * NaN must not leak)
+        const int tok0 = s * kStep;
+        const bool tail = tok0 + kStep > len;
+        if (tail) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (tok0 + 4 * i + g >= len) vreg[i] = u32x4{0u, 0u, 0u, 0u};
+        }
+        lds_order();
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            *reinterpret_cast<u32x4*>(lds + (4 * i + g) * kLdsRow + n * 16) = vreg[i];
+        lds_order();
+
+        // ---- prefetch the next step while this one is being reduced
+        if (s + 1 < s_hi) issue_loads();
+
+        // ---- online softmax, base 2
+        float sv[8];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sv[4 * t + e] = sc[t][e] * a.scale_log2;
+        if (tail) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (tok0 + 4 * i + g >= len) sv[i] = -INFINITY;
+        }
+        float mx = sv[0];
+#pragma unroll
+        for (int i = 1; i < 8; ++i) mx = fmaxf(mx, sv[i]);
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        m_run = m_new;
+        float psum = 0.f;
+        float pv[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            pv[i] = __builtin_amdgcn_exp2f(sv[i] - m_new);
+            psum += pv[i];
+        }
+        l_run = l_run * alpha + psum;
+        bf16x8 pb;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) pb[i] = (__bf16)pv[i];
+        if (__any(alpha != 1.f)) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) acc[t] *= alpha;
+        }
+
+        // ---- O^T += V^T P^T : A operand element i of lane (g, n) is V[token 4 i + g][16 t + n]
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const unsigned char* col = lds + g * kLdsRow + (16 * t + n) * 2;
+            u32x4 vt;
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                uint32_t lo = *reinterpret_cast<const uint16_t*>(col + (8 * p) * kLdsRow);
+                uint32_t hi = *reinterpret_cast<const uint16_t*>(col + (8 * p + 4) * kLdsRow);
+                vt[p] = lo | (hi << 16);
+            }
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vt), pb, acc[t], 0, 0, 0);
+        }
+        lds_order();
+    }
+
+    // ---- leave the partial result of this segment
+    l_run += __shfl_xor(l_run, 16);
+    l_run += __shfl_xor(l_run, 32);
+    const int64_t slot = (int64_t)h * a.slots_per_head + w + b;
+    if (n < G) {
+        float* po = a.po + (slot * G + n) * kD + 4 * g;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) *reinterpret_cast<f32x4*>(po + 16 * t) = acc[t];
+        if (g == 0) {
+            float2 v2 = make_float2(m_run, l_run);
+            *reinterpret_cast<float2*>(a.ml + (slot * G + n) * 2) = v2;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(512) paged_decode_split_kernel(DecodeArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_all[];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int waves = blockDim.x >> 6;
+    const int h = __builtin_amdgcn_readfirstlane(blockIdx.y * waves + wave);
+    const int w = blockIdx.x;
+    const int W = gridDim.x;
+    unsigned char* lds = lds_all + wave * kLdsWave;
+
+    // total number of steps
+    int total = 0;
+    for (int c = 0; c < a.batch; c += 64) {
+        const int i = c + lane;
+        total += wave_sum(i < a.batch ? steps_of(a.ctx[i]) : 0);
+    }
+    total = __builtin_amdgcn_readfirstlane(total);   // wave-uniform: keep the plan in scalar registers
+    int span = (total + W - 1) / W;
+    span = span < kMinSpan ? kMinSpan : span;
+    if (w == 0 && h == 0 && lane == 0) {
+        a.header[0] = W;
+        a.header[1] = span;
+        a.header[2] = total;
+    }
+    const int lo = w * span;
+    const int hi = (lo + span < total) ? lo + span : total;
+    if (lo >= hi) return;
+
+    int running = 0;
+    for (int c = 0; c < a.batch; c += 64) {
+        const int i = c + lane;
+        const int len = i < a.batch ? a.ctx[i] : 0;
+        const int cnt = steps_of(len);
+        const int incl = wave_inclusive_scan(cnt, lane);
+        const int start = running + incl - cnt;
+        const int end = start + cnt;
+        unsigned long long hits = __ballot(cnt > 0 && start < hi && end > lo);
+        while (hits) {
+            const int bit = __builtin_ctzll(hits);
+            hits &= hits - 1;
+            const int st = __builtin_amdgcn_readlane(start, bit);
+            const int en = __builtin_amdgcn_readlane(end, bit);
+            const int ln = __builtin_amdgcn_readlane(len, bit);
+            const int s_lo = (st > lo ? st : lo) - st;
+            const int s_hi = (en < hi ? en : hi) - st;
+            const int b = c + bit;
+            if (h == 0 && lane == 0) {
+                if (s_lo == 0) a.seg_first[b] = w;
+                if (s_hi == en - st) a.seg_last[b] = w;
+            }
+            run_segment(a, lds, b, ln, s_lo, s_hi, h, w, lane);
+        }
+        running += __builtin_amdgcn_readlane(incl, 63);
+        if (running >= hi) break;
+    }
+}
+
+struct MergeArgs {
+    uint16_t* out;
+    int64_t out_stride0;
+    const int32_t* ctx;
+    int group;
+    const int32_t* header;
+    const int32_t* seg_first;
+    const int32_t* seg_last;
+    const float* ml;
+    const float* po;
+    int batch;
+};
+
+// grid (batch, Hkv), 128 threads: thread d folds the segments of (sequence, KV head) for every
+// query head of the group.
+__global__ void __launch_bounds__(128) paged_decode_merge_kernel(MergeArgs a) {
+    const int b = blockIdx.x;
+    const int h = blockIdx.y;
+    const int d = threadIdx.x;
+    const int G = a.group;
+    uint16_t* orow = a.out + (int64_t)b * a.out_stride0 + (int64_t)h * G * kD + d;
+    if (a.ctx[b] <= 0) {
+        for (int n = 0; n < G; ++n) orow[n * kD] = 0;
+        return;
+    }
+    const int W = a.header[0];
+    const int w0 = a.seg_first[b];
+    const int w1 = a.seg_last[b];
+    const int64_t slot0 = (int64_t)h * (W + a.batch) + b;
+    for (int n = 0; n < G; ++n) {
+        float mx = -INFINITY;
+        for (int w = w0; w <= w1; ++w) mx = fmaxf(mx, a.ml[((slot0 + w) * G + n) * 2]);
+        float num = 0.f, den = 0.f;
+        for (int w = w0; w <= w1; ++w) {
+            const float* mlp = a.ml + ((slot0 + w) * G + n) * 2;
+            const float wt = __builtin_amdgcn_exp2f(mlp[0] - mx);
+            den += wt * mlp[1];
+            num += wt * a.po[((slot0 + w) * G + n) * kD + d];
+        }
+        const __bf16 r = (__bf16)(num / den);
+        orow[n * kD] = __builtin_bit_cast(uint16_t, r);
+    }
+}
+
+int g_split_workgroups = 0;
+
+int device_cu_count() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return 256;
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) return 256;
+        cus = v;
+    }
+    return cus;
+}
+
+struct Launch {
+    int waves;      // wavefronts (KV heads) per workgroup
+    int grid_y;
+    int W;
+};
+
+int plan_launch(int64_t hkv, Launch* out) {
+    if (hkv <= 0) return INFER_KV_EINVAL;
+    int waves;
+    if (hkv <= 8) waves = (int)hkv;
+    else if (hkv % 8 == 0) waves = 8;
+    else return INFER_KV_EUNSUPPORTED;
+    int W = g_split_workgroups;
+    if (W <= 0) {
+        W = device_cu_count() * 8 / (int)hkv;   // two wavefronts per SIMD over the whole chip
+        if (W < 1) W = 1;
+    }
+    if (W > INFER_KV_MAX_SPLIT_WG) W = INFER_KV_MAX_SPLIT_WG;
+    out->waves = waves;
+    out->grid_y = (int)(hkv / waves);
+    out->W = W;
+    return INFER_KV_OK;
+}
+
+int check_shape(int64_t batch, int64_t hq, int64_t hkv, int64_t d, int64_t bs, int64_t nblk) {
+    if (batch <= 0 || hq <= 0 || hkv <= 0 || nblk <= 0 || bs <= 0) return INFER_KV_EINVAL;
+    if (batch > (1 << 20)) return INFER_KV_EINVAL;
+    if (d != kD) return INFER_KV_EUNSUPPORTED;
+    if (hq % hkv != 0 || hq / hkv > 16) return INFER_KV_EUNSUPPORTED;
+    if (bs % kStep != 0) return INFER_KV_EUNSUPPORTED;
+    return INFER_KV_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t infer_paged_decode_workspace_bytes(int64_t max_batch, int64_t num_q_heads, int64_t num_kv_heads,
+                                          int64_t head_dim) {
+    if (max_batch <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 || head_dim != kD) return 0;
+    if (num_q_heads % num_kv_heads != 0) return 0;
+    DecodeWorkspace ws = decode_workspace_layout(max_batch, num_q_heads / num_kv_heads, num_kv_heads);
+    return ws.total_bytes;
+}
+
+int infer_paged_decode_set_split_workgroups(int workgroups) {
+    int prev = g_split_workgroups;
+    g_split_workgroups = workgroups < 0 ? 0 : workgroups;
+    return prev;
+}
+
+int infer_paged_decode_split_bf16(const void* q, int64_t q_stride0, const void* k_cache, const void* v_cache,
+                                  int64_t cache_block_stride, int64_t cache_token_stride,
+                                  const int32_t* block_table, int64_t bt_stride0, const int32_t* context_lens,
+                                  int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                                  int64_t block_size, int64_t num_blocks, float scale, void* workspace,
+                                  size_t workspace_bytes, void* stream) {
+    if (!q || !k_cache || !v_cache || !block_table || !context_lens || !workspace) return INFER_KV_EINVAL;
+    int rc = check_shape(batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks);
+    if (rc) return rc;
+    // 16-byte vector loads: every row start must be 16-byte aligned.
+    if (((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)workspace) & 15) return INFER_KV_EALIGN;
+    if ((q_stride0 | cache_block_stride | cache_token_stride) & 7) return INFER_KV_EALIGN;
+    if (cache_token_stride < num_kv_heads * kD || cache_block_stride < block_size * cache_token_stride) return INFER_KV_EINVAL;
+    // lane offsets inside one step are kept in 32 bits
+    if (32 * cache_token_stride >= (int64_t)1 << 31) return INFER_KV_EINVAL;
+    Launch L;
+    rc = plan_launch(num_kv_heads, &L);
+    if (rc) return rc;
+    const int G = (int)(num_q_heads / num_kv_heads);
+    DecodeWorkspace ws = decode_workspace_layout(batch, G, num_kv_heads);
+    if (ws.total_bytes > workspace_bytes) return INFER_KV_EWORKSPACE;
+
+    DecodeArgs a;
+    a.q = (const uint16_t*)q;
+    a.q_stride0 = q_stride0;
+    a.k = (const uint16_t*)k_cache;
+    a.v = (const uint16_t*)v_cache;
+    a.blk_stride = cache_block_stride;
+    a.tok_stride = cache_token_stride;
+    a.bt = block_table;
+    a.bt_stride0 = bt_stride0;
+    a.ctx = context_lens;
+    a.batch = (int)batch;
+    a.group = G;
+    a.num_kv_heads = (int)num_kv_heads;
+    a.block_size = (int)block_size;
+    a.num_blocks = (int)num_blocks;
+    a.scale_log2 = scale * 1.4426950408889634f;
+    char* base = (char*)workspace;
+    a.header = (int32_t*)(base + ws.header_off);
+    a.seg_first = (int32_t*)(base + ws.seg_first_off);
+    a.seg_last = (int32_t*)(base + ws.seg_last_off);
+    a.ml = (float*)(base + ws.ml_off);
+    a.po = (float*)(base + ws.po_off);
+    a.slots_per_head = L.W + (int)batch;
+
+    const size_t lds_bytes = (size_t)L.waves * kLdsWave;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)paged_decode_split_kernel,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 8 * kLdsWave);
+        if (e != hipSuccess) return (int)e;
+        attr_set = true;
+    }
+    dim3 grid(L.W, L.grid_y, 1), block(64 * L.waves, 1, 1);
+    hipLaunchKernelGGL(paged_decode_split_kernel, grid, block, lds_bytes, (hipStream_t)stream, a);
+    return (int)hipGetLastError();
+}
+
+int infer_paged_decode_merge_bf16(void* out, int64_t out_stride0, const int32_t* context_lens, int64_t batch,
+                                  int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                                  const void* workspace, size_t workspace_bytes, void* stream) {
+    if (!out || !context_lens || !workspace) return INFER_KV_EINVAL;
+    if (batch <= 0 || num_q_heads <= 0 || num_kv_heads <= 0) return INFER_KV_EINVAL;
+    if (head_dim != kD) return INFER_KV_EUNSUPPORTED;
+    if (num_q_heads % num_kv_heads != 0 || num_q_heads / num_kv_heads > 16) return INFER_KV_EUNSUPPORTED;
+    if (out_stride0 < num_q_heads * kD) return INFER_KV_EINVAL;
+    const int G = (int)(num_q_heads / num_kv_heads);
+    DecodeWorkspace ws = decode_workspace_layout(batch, G, num_kv_heads);
+    if (ws.total_bytes > workspace_bytes) return INFER_KV_EWORKSPACE;
+    const char* base = (const char*)workspace;
+    MergeArgs m;
+    m.out = (uint16_t*)out;
+    m.out_stride0 = out_stride0;
+    m.ctx = context_lens;
+    m.group = G;
+    m.header = (const int32_t*)(base + ws.header_off);
+    m.seg_first = (const int32_t*)(base + ws.seg_first_off);
+    m.seg_last = (const int32_t*)(base + ws.seg_last_off);
+    m.ml = (const float*)(base + ws.ml_off);
+    m.po = (const float*)(base + ws.po_off);
+    m.batch = (int)batch;
+    dim3 grid((unsigned)batch, (unsigned)num_kv_heads, 1), block(128, 1, 1);
+    hipLaunchKernelGGL(paged_decode_merge_kernel, grid, block, 0, (hipStream_t)stream, m);
+    return (int)hipGetLastError();
+}
+
+int infer_paged_decode_bf16(const void* q, int64_t q_stride0, const void* k_cache, const void* v_cache,
+                            int64_t cache_block_stride, int64_t cache_token_stride, void* out,
+                            int64_t out_stride0, const int32_t* block_table, int64_t bt_stride0,
+                            const int32_t* context_lens, int64_t batch, int64_t num_q_heads,
+                            int64_t num_kv_heads, int64_t head_dim, int64_t block_size, int64_t num_blocks,
+                            float scale, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!out) return INFER_KV_EINVAL;
+    int rc = infer_paged_decode_split_bf16(q, q_stride0, k_cache, v_cache, cache_block_stride, cache_token_stride,
+                                           block_table, bt_stride0, context_lens, batch, num_q_heads,
+                                           num_kv_heads, head_dim, block_size, num_blocks, scale, workspace,
+                                           workspace_bytes, stream);
+    if (rc) return rc;
+    return infer_paged_decode_merge_bf16(out, out_stride0, context_lens, batch, num_q_heads, num_kv_heads,
+                                         head_dim, workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"

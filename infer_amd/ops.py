@@ -1,0 +1,146 @@
+"""Python entry points of the paged KV-cache path, argument-compatible with the reference.
+
+* ``store_kvcache``            - same signature and asserts as ``infer/ops/attention.py:38-45``.
+* ``flash_attn_with_kvcache``  - keyword set used at ``infer/ops/attention.py:118-120``.
+* ``flash_attn_decode``        - the signature the stub ``src/operators/flashattn/flashattn_decode.cu:11-12``
+  intended: ``(Q, K, V, is_causal, block_table, O)`` with an out-parameter, plus the context lengths
+  it forgot.
+
+All of them launch hand-written HIP kernels through the C ABI of ``libinfer_kv.so`` on torch's
+current stream.  Tensors must live on the GPU; there is no CPU path.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+_workspaces: dict = {}
+
+
+def _stream_ptr(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _require_gpu(*tensors):
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError("infer_amd ops need GPU tensors: the HIP kernels are the only implementation")
+
+
+def store_kvcache(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                  slot_mapping: torch.Tensor) -> None:
+    """Scatter ``key``/``value`` rows ``[N, Hkv, D]`` into the paged caches at ``slot_mapping``.
+
+    Rows with a negative slot are skipped.  Bit-exact copy."""
+    n, num_heads, head_dim = key.shape
+    d = num_heads * head_dim
+    assert key.stride(-1) == 1 and value.stride(-1) == 1
+    assert key.stride(1) == head_dim and value.stride(1) == head_dim
+    assert k_cache.stride(1) == d and v_cache.stride(1) == d
+    assert slot_mapping.numel() == n
+    assert key.dtype == torch.bfloat16 and value.dtype == torch.bfloat16
+    assert k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16
+    assert slot_mapping.dtype == torch.int32 and slot_mapping.is_contiguous()
+    assert value.shape == key.shape
+    _require_gpu(key, value, k_cache, v_cache, slot_mapping)
+    assert k_cache.stride(0) == k_cache.shape[1] * d and v_cache.stride(0) == v_cache.shape[1] * d
+    if n == 0:
+        return
+    num_slots = k_cache.shape[0] * k_cache.shape[1]
+    lib = _lib.load()
+    rc = lib.infer_kv_append_bf16(key.data_ptr(), key.stride(0), value.data_ptr(), value.stride(0),
+                                  k_cache.data_ptr(), v_cache.data_ptr(), slot_mapping.data_ptr(),
+                                  n, d, num_slots, _stream_ptr(key))
+    _lib.check(rc, "store_kvcache")
+
+
+def decode_workspace(device, max_batch: int, num_q_heads: int, num_kv_heads: int, head_dim: int) -> torch.Tensor:
+    """Workspace for the split-KV partial results, cached per (device, shape): allocated once so that
+    steady-state decode steps (and HIP graph replays) never allocate."""
+    key = (str(device), num_q_heads, num_kv_heads, head_dim)
+    ws = _workspaces.get(key)
+    if ws is None or ws[0] < max_batch:
+        cap = max(max_batch, 64 if ws is None else 2 * ws[0])
+        nbytes = _lib.load().infer_paged_decode_workspace_bytes(cap, num_q_heads, num_kv_heads, head_dim)
+        if nbytes == 0:
+            raise RuntimeError("paged decode: unsupported shape "
+                               f"(Hq={num_q_heads}, Hkv={num_kv_heads}, D={head_dim})")
+        ws = (cap, torch.empty(nbytes, dtype=torch.uint8, device=device))
+        _workspaces[key] = ws
+    return ws[1]
+
+
+def _decode_args(q3, k_cache, v_cache, cache_seqlens, block_table):
+    assert q3.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16
+    assert cache_seqlens.dtype == torch.int32 and block_table.dtype == torch.int32
+    assert k_cache.dim() == 4 and k_cache.shape == v_cache.shape
+    assert k_cache.stride() == v_cache.stride()
+    b, hq, d = q3.shape
+    nblk, bs, hkv, dk = k_cache.shape
+    assert dk == d and q3.stride(2) == 1 and q3.stride(1) == d
+    assert k_cache.stride(3) == 1 and k_cache.stride(2) == d
+    assert cache_seqlens.numel() == b and cache_seqlens.is_contiguous()
+    assert block_table.shape[0] == b and block_table.stride(1) == 1
+    _require_gpu(q3, k_cache, v_cache, cache_seqlens, block_table)
+    return b, hq, d, nblk, bs, hkv
+
+
+def paged_attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                      context_lens: torch.Tensor, scale: float, out: torch.Tensor, workspace=None) -> None:
+    """Out-parameter form: ``q``/``out`` are ``[B, Hq, D]``."""
+    b, hq, d, nblk, bs, hkv = _decode_args(q, k_cache, v_cache, context_lens, block_table)
+    assert out.shape == q.shape and out.dtype == torch.bfloat16 and out.stride(2) == 1 and out.stride(1) == d
+    if workspace is None:
+        workspace = decode_workspace(q.device, b, hq, hkv, d)
+    lib = _lib.load()
+    rc = lib.infer_paged_decode_bf16(
+        q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), k_cache.stride(0), k_cache.stride(1),
+        out.data_ptr(), out.stride(0), block_table.data_ptr(), block_table.stride(0), context_lens.data_ptr(),
+        b, hq, hkv, d, bs, nblk, float(scale), workspace.data_ptr(), workspace.numel(), _stream_ptr(q))
+    _lib.check(rc, "paged_attn_decode")
+
+
+def paged_attn_decode_split(q, k_cache, v_cache, block_table, context_lens, scale, workspace) -> None:
+    """Bandwidth-bound phase alone (partials stay in ``workspace``); for profiling."""
+    b, hq, d, nblk, bs, hkv = _decode_args(q, k_cache, v_cache, context_lens, block_table)
+    rc = _lib.load().infer_paged_decode_split_bf16(
+        q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), k_cache.stride(0), k_cache.stride(1),
+        block_table.data_ptr(), block_table.stride(0), context_lens.data_ptr(),
+        b, hq, hkv, d, bs, nblk, float(scale), workspace.data_ptr(), workspace.numel(), _stream_ptr(q))
+    _lib.check(rc, "paged_attn_decode_split")
+
+
+def paged_attn_decode_merge(out, context_lens, num_kv_heads, workspace) -> None:
+    b, hq, d = out.shape
+    rc = _lib.load().infer_paged_decode_merge_bf16(
+        out.data_ptr(), out.stride(0), context_lens.data_ptr(), b, hq, num_kv_heads, d,
+        workspace.data_ptr(), workspace.numel(), _stream_ptr(out))
+    _lib.check(rc, "paged_attn_decode_merge")
+
+
+def flash_attn_with_kvcache(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, *,
+                            cache_seqlens: torch.Tensor, block_table: torch.Tensor,
+                            softmax_scale: float | None = None, causal: bool = True) -> torch.Tensor:
+    """``q`` is ``[B, 1, Hq, D]``; returns ``[B, 1, Hq, D]``.  With a single query token the causal
+    mask hides nothing, so ``causal`` only has to be accepted."""
+    assert q.dim() == 4 and q.shape[1] == 1, "decode takes one query token per sequence"
+    if softmax_scale is None:
+        softmax_scale = q.shape[-1] ** -0.5
+    q3 = q[:, 0]
+    out = torch.empty((q.shape[0], q.shape[2], q.shape[3]), dtype=q.dtype, device=q.device)
+    paged_attn_decode(q3, k_cache, v_cache, block_table, cache_seqlens, softmax_scale, out)
+    return out.unsqueeze(1)
+
+
+def flash_attn_decode(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, is_causal: bool,
+                      block_table: torch.Tensor, O: torch.Tensor, context_lens: torch.Tensor,
+                      softmax_scale: float | None = None) -> None:
+    """``Q``/``O`` ``[B, Hq, D]``, ``K``/``V`` the paged caches."""
+    if softmax_scale is None:
+        softmax_scale = Q.shape[-1] ** -0.5
+    paged_attn_decode(Q, K, V, block_table, context_lens, softmax_scale, O)
+
+
+def set_split_workgroups(n: int) -> int:
+    return _lib.load().infer_paged_decode_set_split_workgroups(int(n))

@@ -1,0 +1,106 @@
+"""KV append on the GPU against the oracle: bit-exact (pure copy)."""
+import numpy as np
+import pytest
+import torch
+
+from infer_amd import ops, workloads
+from oracle import paged_ref
+from tests.helpers import bits
+
+pytestmark = pytest.mark.gpu
+
+
+def run_both(key, value, k_cache, v_cache, slots):
+    """Runs the HIP append on copies of the caches and the oracle on host copies; returns both."""
+    kc, vc = k_cache.clone(), v_cache.clone()
+    ops.store_kvcache(key, value, kc, vc, slots)
+    torch.cuda.synchronize()
+    ek, ev = bits(k_cache).copy(), bits(v_cache).copy()
+    paged_ref.append_ref(bits(key), bits(value), ek, ev, slots.cpu().numpy())
+    return bits(kc), bits(vc), ek, ev
+
+
+def test_cfg1_decode_rows(gpu):
+    wl = workloads.cfg1().to(gpu)
+    gk, gv, ek, ev = run_both(wl.k_new, wl.v_new, wl.k_cache, wl.v_cache, wl.slot_mapping)
+    assert np.array_equal(gk, ek) and np.array_equal(gv, ev)
+    # and the new rows really are where the block table says the newest token lives
+    for i, n in enumerate(wl.lengths):
+        blk = int(wl.block_table[i, (n - 1) // 256])
+        assert np.array_equal(gk[blk, (n - 1) % 256], bits(wl.k_new)[i])
+
+
+def test_cfg3_prefill_rows_with_padding(gpu):
+    wl = workloads.cfg3().to(gpu)
+    assert int((wl.slot_mapping < 0).sum()) > 0
+    gk, gv, ek, ev = run_both(wl.k_new, wl.v_new, wl.k_cache, wl.v_cache, wl.slot_mapping)
+    assert np.array_equal(gk, ek) and np.array_equal(gv, ev)
+
+
+def test_strided_rows_from_fused_qkv(gpu):
+    """K and V are views of one qkv projection (row stride (Hq + 2 Hkv) D), as in
+    infer/models/Qwen3.py:110-111."""
+    g = torch.Generator(device="cpu").manual_seed(3)
+    hq, hkv, d, n = 32, 8, 128, 77
+    qkv = torch.randn((n, (hq + 2 * hkv) * d), generator=g).to(torch.bfloat16).to(gpu)
+    _, k, v = qkv.split([hq * d, hkv * d, hkv * d], dim=-1)
+    k, v = k.view(n, hkv, d), v.view(n, hkv, d)
+    assert not k.is_contiguous()
+    cache = torch.randn((2, 6, 256, hkv, d), generator=g).to(torch.bfloat16).to(gpu)
+    slots = torch.randperm(6 * 256, generator=g)[:n].to(torch.int32).to(gpu)
+    gk, gv, ek, ev = run_both(k, v, cache[0], cache[1], slots)
+    assert np.array_equal(gk, ek) and np.array_equal(gv, ev)
+
+
+@pytest.mark.parametrize("hkv,d", [(1, 64), (2, 128), (4, 128), (8, 64), (8, 128), (16, 128), (3, 40)])
+def test_row_widths(gpu, hkv, d):
+    g = torch.Generator(device="cpu").manual_seed(hkv * 131 + d)
+    n, nblk, bs = 53, 3, 64
+    key = torch.randn((n, hkv, d), generator=g).to(torch.bfloat16).to(gpu)
+    val = torch.randn((n, hkv, d), generator=g).to(torch.bfloat16).to(gpu)
+    kc = torch.randn((nblk, bs, hkv, d), generator=g).to(torch.bfloat16).to(gpu)
+    vc = torch.randn((nblk, bs, hkv, d), generator=g).to(torch.bfloat16).to(gpu)
+    slots = torch.randperm(nblk * bs, generator=g)[:n].to(torch.int32)
+    slots[::7] = -1
+    gk, gv, ek, ev = run_both(key, val, kc, vc, slots.to(gpu))
+    assert np.array_equal(gk, ek) and np.array_equal(gv, ev)
+
+
+def test_all_padding_and_empty(gpu):
+    hkv, d = 8, 128
+    kc = torch.zeros((2, 256, hkv, d), dtype=torch.bfloat16, device=gpu)
+    vc = torch.zeros_like(kc)
+    key = torch.ones((5, hkv, d), dtype=torch.bfloat16, device=gpu)
+    ops.store_kvcache(key, key, kc, vc, torch.full((5,), -1, dtype=torch.int32, device=gpu))
+    ops.store_kvcache(key[:0], key[:0], kc, vc, torch.zeros((0,), dtype=torch.int32, device=gpu))
+    torch.cuda.synchronize()
+    assert not kc.any() and not vc.any()
+
+
+def test_out_of_range_slot_is_skipped(gpu):
+    hkv, d = 8, 128
+    kc = torch.zeros((1, 256, hkv, d), dtype=torch.bfloat16, device=gpu)
+    vc = torch.zeros_like(kc)
+    key = torch.ones((3, hkv, d), dtype=torch.bfloat16, device=gpu)
+    slots = torch.tensor([255, 256, 1 << 30], dtype=torch.int32, device=gpu)
+    ops.store_kvcache(key, key, kc, vc, slots)
+    torch.cuda.synchronize()
+    assert bool(kc[0, 255].eq(1).all()) and int(kc.ne(0).sum()) == hkv * d
+
+
+def test_scatter_then_gather_roundtrip_full_size(gpu):
+    """Size-independent property at cfg3 scale: after the append, reading the caches back through
+    slot_mapping returns exactly the appended rows, and every other cache row is untouched."""
+    wl = workloads.cfg3().to(gpu)
+    kc, vc = wl.k_cache.clone(), wl.v_cache.clone()
+    ops.store_kvcache(wl.k_new, wl.v_new, kc, vc, wl.slot_mapping)
+    torch.cuda.synchronize()
+    valid = wl.slot_mapping >= 0
+    rows = wl.slot_mapping[valid].long()
+    width = wl.num_kv_heads * wl.head_dim
+    assert torch.equal(kc.view(-1, width)[rows], wl.k_new[valid].reshape(-1, width))
+    assert torch.equal(vc.view(-1, width)[rows], wl.v_new[valid].reshape(-1, width))
+    untouched = torch.ones(kc.shape[0] * kc.shape[1], dtype=torch.bool, device=gpu)
+    untouched[rows] = False
+    assert torch.equal(kc.view(-1, width)[untouched], wl.k_cache.view(-1, width)[untouched])
+    assert torch.equal(vc.view(-1, width)[untouched], wl.v_cache.view(-1, width)[untouched])

@@ -1,0 +1,173 @@
+"""Paged decode attention on the GPU against the fp32 CPU oracle.
+
+Bar: max abs error of the bf16 output <= 2e-2 against the fp32 oracle (tests/helpers.ATTN_ATOL)."""
+import numpy as np
+import pytest
+import torch
+
+from infer_amd import ops, workloads
+from tests.helpers import ATTN_ATOL, bits, f32, oracle_decode
+
+pytestmark = pytest.mark.gpu
+
+
+def gpu_decode(wl, splits=None):
+    if splits is not None:
+        prev = ops.set_split_workgroups(splits)
+    try:
+        out = ops.flash_attn_with_kvcache(wl.q.unsqueeze(1), wl.k_cache, wl.v_cache,
+                                          cache_seqlens=wl.context_lens, block_table=wl.block_table,
+                                          softmax_scale=wl.scale, causal=True)
+        torch.cuda.synchronize()
+    finally:
+        if splits is not None:
+            ops.set_split_workgroups(prev)
+    return out[:, 0]
+
+
+def check(wl, splits=None, atol=ATTN_ATOL):
+    got = f32(gpu_decode(wl, splits))
+    want = oracle_decode(wl)
+    err = float(np.abs(got - want).max())
+    assert np.isfinite(got).all()
+    assert err <= atol, f"{wl.name}: max abs err {err}"
+    return err
+
+
+def test_cfg1_append_then_decode(gpu):
+    """The reference's step order (infer/ops/attention.py:108-120): append the new row, then attend."""
+    wl = workloads.cfg1().to(gpu)
+    ops.store_kvcache(wl.k_new, wl.v_new, wl.k_cache, wl.v_cache, wl.slot_mapping)
+    err = check(wl)
+    print("cfg1 max abs err", err)
+
+
+@pytest.mark.parametrize("splits", [1, 3, 64, 1024])
+def test_split_count_invariance(gpu, splits):
+    wl = workloads.cfg1().to(gpu)
+    check(wl, splits=splits)
+
+
+@pytest.mark.parametrize("hq,hkv", [(8, 8), (16, 8), (32, 8), (64, 8), (4, 1), (8, 2), (32, 4), (32, 16), (16, 1)])
+def test_group_sizes_and_head_counts(gpu, hq, hkv):
+    wl = workloads.make_decode_workload(f"g{hq}-{hkv}", [1, 31, 32, 33, 255, 256, 257, 600], hq, hkv,
+                                        seed=hq * 7 + hkv).to(gpu)
+    check(wl)
+
+
+@pytest.mark.parametrize("bs", [32, 64, 128, 256, 512])
+def test_block_sizes(gpu, bs):
+    wl = workloads.make_decode_workload(f"bs{bs}", [5, 97, 511, 512, 513, 1300], 32, 8, bs=bs, seed=bs).to(gpu)
+    check(wl)
+
+
+def test_single_token_returns_v(gpu):
+    """L = 1: softmax over one key is 1, so O = V[0] exactly (bf16 round trip)."""
+    wl = workloads.make_decode_workload("one", [1, 1, 1], 32, 8, seed=5).to(gpu)
+    got = gpu_decode(wl)
+    for i in range(3):
+        v0 = wl.v_cache[int(wl.block_table[i, 0]), 0]                    # [Hkv, D]
+        assert torch.equal(got[i], v0.repeat_interleave(4, dim=0))
+
+
+def test_equal_keys_give_mean_of_values(gpu):
+    wl = workloads.make_decode_workload("mean", [300, 64], 16, 8, seed=6).to(gpu)
+    wl.k_cache[:] = wl.k_cache[0, 0]          # every key identical -> uniform softmax
+    got = f32(gpu_decode(wl))
+    for i, n in enumerate(wl.lengths):
+        rows = torch.cat([wl.v_cache[int(b)] for b in wl.block_table[i, : (n + 255) // 256]])[:n]
+        mean = rows.float().mean(dim=0).cpu().numpy()                    # [Hkv, D]
+        assert np.abs(got[i] - np.repeat(mean, 2, axis=0)).max() <= 1e-2
+
+
+def test_block_permutation_invariance(gpu):
+    """Same logical tokens under a different physical placement give bit-identical output."""
+    wl = workloads.make_decode_workload("perm", [700, 1023, 40], 32, 8, nblk=32, seed=7).to(gpu)
+    a = gpu_decode(wl)
+    perm = torch.randperm(32, generator=torch.Generator().manual_seed(1)).to(gpu)
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(32, device=gpu)
+    kc2, vc2 = wl.k_cache[perm], wl.v_cache[perm]      # new block j holds old block perm[j]
+    bt2 = torch.where(wl.block_table >= 0, inv[wl.block_table.clamp(min=0).long()].int(), wl.block_table)
+    out = ops.flash_attn_with_kvcache(wl.q.unsqueeze(1), kc2, vc2, cache_seqlens=wl.context_lens,
+                                      block_table=bt2, softmax_scale=wl.scale)[:, 0]
+    assert torch.equal(a, out)
+
+
+def test_zero_length_rows_and_graph_padding(gpu):
+    """Rows with context_len 0 (the reference zero-fills its graph buffers:
+    infer/engine/model_runner.py:144-146) give zeros and do not disturb their neighbours; unused
+    table entries may hold -1 or garbage."""
+    wl = workloads.make_decode_workload("pad", [300, 1, 513, 77], 32, 8, seed=8).to(gpu)
+    ctx = wl.context_lens.clone()
+    ctx[1] = 0
+    bt = wl.block_table.clone()
+    bt[bt < 0] = 10_000_000           # must never be dereferenced
+    bt[1] = -1
+    out = ops.flash_attn_with_kvcache(wl.q.unsqueeze(1), wl.k_cache, wl.v_cache, cache_seqlens=ctx,
+                                      block_table=bt, softmax_scale=wl.scale)[:, 0]
+    torch.cuda.synchronize()
+    want = oracle_decode(wl)
+    got = f32(out)
+    assert not got[1].any()
+    for i in (0, 2, 3):
+        assert np.abs(got[i] - want[i]).max() <= ATTN_ATOL
+    ctx[:] = 0
+    out = ops.flash_attn_with_kvcache(wl.q.unsqueeze(1), wl.k_cache, wl.v_cache, cache_seqlens=ctx,
+                                      block_table=bt, softmax_scale=wl.scale)
+    assert not out.any()
+
+
+def test_stale_nan_beyond_length_is_ignored(gpu):
+    """Cache rows past a sequence's length may hold anything (a freed sequence's data, NaN bit
+    patterns of never-written memory): they must not reach the output."""
+    wl = workloads.make_decode_workload("nan", [37, 289, 1000], 32, 8, seed=9).to(gpu)
+    want = oracle_decode(wl)
+    for i, n in enumerate(wl.lengths):
+        blk = int(wl.block_table[i, (n - 1) // 256])
+        wl.k_cache[blk, n % 256 or 256:] = float("nan")
+        wl.v_cache[blk, n % 256 or 256:] = float("nan")
+    got = f32(gpu_decode(wl))
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= ATTN_ATOL
+
+
+def test_large_batch(gpu):
+    g = torch.Generator().manual_seed(11)
+    lens = torch.randint(1, 700, (300,), generator=g).tolist()
+    wl = workloads.make_decode_workload("b300", lens, 16, 8, seed=11).to(gpu)
+    check(wl)
+
+
+def test_cfg2_full_size(gpu):
+    wl = workloads.cfg2(device=gpu)
+    err = check(wl)
+    print("cfg2 max abs err", err)
+
+
+def test_cfg4_long_context(gpu):
+    wl = workloads.cfg4(device=gpu)
+    err = check(wl)
+    print("cfg4 max abs err", err)
+
+
+def test_layer_view_of_fused_cache(gpu):
+    """Caches as per-layer views of one [2, layers, nblk, bs, Hkv, D] tensor
+    (infer/engine/model_runner.py:58-64)."""
+    wl = workloads.make_decode_workload("layers", [400, 90], 32, 8, nblk=6, seed=12).to(gpu)
+    big = torch.zeros((2, 3, 6, 256, 8, 128), dtype=torch.bfloat16, device=gpu)
+    big[0, 1], big[1, 1] = wl.k_cache, wl.v_cache
+    out = ops.flash_attn_with_kvcache(wl.q.unsqueeze(1), big[0, 1], big[1, 1], cache_seqlens=wl.context_lens,
+                                      block_table=wl.block_table, softmax_scale=wl.scale)[:, 0]
+    assert np.abs(f32(out) - oracle_decode(wl)).max() <= ATTN_ATOL
+
+
+def test_errors_are_loud(gpu):
+    wl = workloads.make_decode_workload("err", [10], 32, 8, seed=1).to(gpu)
+    with pytest.raises(RuntimeError):
+        ops.flash_attn_with_kvcache(wl.q.cpu().unsqueeze(1), wl.k_cache, wl.v_cache,
+                                    cache_seqlens=wl.context_lens, block_table=wl.block_table)
+    q64 = torch.zeros((1, 1, 32, 64), dtype=torch.bfloat16, device=gpu)
+    kc = torch.zeros((2, 256, 8, 64), dtype=torch.bfloat16, device=gpu)
+    with pytest.raises(RuntimeError):
+        ops.flash_attn_with_kvcache(q64, kc, kc, cache_seqlens=wl.context_lens, block_table=wl.block_table)
