@@ -10,7 +10,8 @@ import os
 import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libinfer_kv.so")
+# INFER_KV_LIB lets a developer point at an experimental build of the same library.
+LIB_PATH = os.environ.get("INFER_KV_LIB") or os.path.join(_HERE, "libinfer_kv.so")
 
 _lock = threading.Lock()
 _lib = None

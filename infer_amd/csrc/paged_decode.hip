@@ -26,6 +26,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "decode_layout.h"
 
 namespace {
@@ -93,20 +95,104 @@ __device__ __forceinline__ int wave_inclusive_scan(int x, int lane) {
 // write -> read -> write sequence on the private tile needs.
 __device__ __forceinline__ void lds_order() { __asm__ volatile("" ::: "memory"); }
 
-// One (sequence, span) piece: steps [s_lo, s_hi) of sequence b for KV head h.
-__device__ __forceinline__ void run_segment(const DecodeArgs& a, unsigned char* lds, int b, int len,
-                                            int s_lo, int s_hi, int h, int w, int lane) {
+// ---------------------------------------------------------------------------------------------
+// Span plan.  A wavefront first lists the segments (pieces of sequences) of its span in a small
+// wave-private LDS table and gathers the block ids of all of them into ONE vector register
+// (lane i = i-th block touched by the span, "block ordinal" i).  After that the streaming loop
+// needs no memory access for addressing: crossing a block or a sequence boundary is a register
+// read, so loads for the next sequence are in flight long before the current one is finished.
+constexpr int kPlanInts = 8;        // ints per segment record
+constexpr int kMaxSegs = 32;        // segments per batch (a span with more is run in several batches)
+constexpr int kPlanBytes = kMaxSegs * kPlanInts * 4;
+constexpr int kLdsPerWave = kLdsWave + kPlanBytes;
+
+struct SegRec {      // one record of the plan, all wave-uniform
+    int b;           // sequence
+    int len;         // its context length
+    int s_lo, s_hi;  // steps of the sequence covered by this span
+    int ord0;        // block ordinal of the first step's block
+    int in0;         // step index of s_lo inside its block
+    int blk0;        // index of that block in the sequence's table row
+};
+
+__device__ __forceinline__ SegRec read_rec(const int* plan, int seg) {
+    const int* p = plan + seg * kPlanInts;
+    SegRec r;
+    r.b = __builtin_amdgcn_readfirstlane(p[0]);
+    r.len = __builtin_amdgcn_readfirstlane(p[1]);
+    r.s_lo = __builtin_amdgcn_readfirstlane(p[2]);
+    r.s_hi = __builtin_amdgcn_readfirstlane(p[3]);
+    r.ord0 = __builtin_amdgcn_readfirstlane(p[4]);
+    r.in0 = __builtin_amdgcn_readfirstlane(p[5]);
+    r.blk0 = __builtin_amdgcn_readfirstlane(p[6]);
+    return r;
+}
+
+// Walks the steps of a batch of segments in order.  Used three times: by the K loads (two steps
+// ahead), the V loads (one step ahead) and the arithmetic.
+struct StepCursor {
+    int seg, nseg;
+    int s, s_hi;     // current step of the current segment, end of the segment
+    int in, ord;     // step inside its block, block ordinal
+    int b, blk0, ord0;
+    __device__ __forceinline__ void enter(const int* plan, int seg_) {
+        seg = seg_;
+        if (seg < nseg) {
+            const SegRec r = read_rec(plan, seg);
+            s = r.s_lo; s_hi = r.s_hi; in = r.in0; ord = r.ord0; b = r.b; blk0 = r.blk0; ord0 = r.ord0;
+        }
+    }
+    __device__ __forceinline__ bool live() const { return seg < nseg; }
+    __device__ __forceinline__ void advance(const int* plan, int steps_per_blk) {
+        ++s;
+        if (++in == steps_per_blk) { in = 0; ++ord; }
+        if (s == s_hi) enter(plan, seg + 1);
+    }
+};
+
+// Runs one batch of segments for KV head h.
+//
+// Software pipeline (loads return in issue order, so the waits are exact counts): K fragments are
+// double-buffered in registers, V rows single-buffered; while step i is being reduced, K(i+1),
+// then K(i+2) and V(i+1) are in flight, across sequence boundaries.  Loads past the end of the
+// batch are redirected to one dummy 16-byte location instead of being skipped, which keeps the
+// number of outstanding loads at every wait independent of control flow.
+__device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* lds, const int* plan, int nseg,
+                                          int total_steps, int tblv, int h, int w, int lane) {
     const int g = lane >> 4;   // lane group: the k-slice of MFMA operands, the row-quad of results
     const int n = lane & 15;   // operand row / result column
     const int G = a.group;
+    const int steps_per_blk = a.block_size / kStep;
+
+    auto block_id = [&](const StepCursor& c) -> int {
+        int blk;
+        if (c.ord < 64) blk = __builtin_amdgcn_readlane(tblv, c.ord);
+        else   // a single segment longer than 64 blocks (it is alone in its batch)
+            blk = __builtin_amdgcn_readfirstlane(a.bt[(int64_t)c.b * a.bt_stride0 + c.blk0 + (c.ord - c.ord0)]);
+        return blk < 0 ? 0 : (blk >= a.num_blocks ? a.num_blocks - 1 : blk);
+    };
 
     // Q as the B operand of S^T = K Q^T: lane (g, n) holds Q[head n][32 j + 8 g .. +8].
-    bf16x8 qreg[4];
-    {
-        u32x4 z = {0u, 0u, 0u, 0u};
+    auto load_q = [&](int b, u32x4 (&dst)[4]) {
+        const u32x4 z = {0u, 0u, 0u, 0u};
         const uint16_t* qp = a.q + (int64_t)b * a.q_stride0 + (int64_t)(h * G + (n < G ? n : 0)) * kD + 8 * g;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) qreg[j] = as_bf16x8(n < G ? load16(qp + 32 * j) : z);
+        for (int j = 0; j < 4; ++j) dst[j] = n < G ? load16(qp + 32 * j) : z;
+    };
+
+    StepCursor ccur, kcur, vcur;
+    ccur.nseg = kcur.nseg = vcur.nseg = nseg;
+    ccur.enter(plan, 0);
+    kcur = ccur;
+    vcur = ccur;
+    SegRec cseg = read_rec(plan, 0);
+
+    u32x4 qreg[4], qnext[4];
+    load_q(cseg.b, qreg);
+    if (nseg > 1) load_q(__builtin_amdgcn_readfirstlane(plan[kPlanInts]), qnext);
+    else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) qnext[j] = u32x4{0u, 0u, 0u, 0u};
     }
 
     f32x4 acc[8];
@@ -115,52 +201,64 @@ __device__ __forceinline__ void run_segment(const DecodeArgs& a, unsigned char* 
     float m_run = -INFINITY;
     float l_run = 0.f;
 
-    // Block ids of the segment: lane i keeps the table entry of block (tbl_base + i), so the
-    // per-step lookup is a register read instead of a dependent memory load.
-    const int32_t* btrow = a.bt + (int64_t)b * a.bt_stride0;
-    const int steps_per_blk = a.block_size / kStep;
-    const int blk_last = (s_hi - 1) / steps_per_blk;
-    int tbl_base = s_lo / steps_per_blk;
-    int tblv = (tbl_base + lane <= blk_last) ? btrow[tbl_base + lane] : 0;
-    int nxt_bi = tbl_base;                       // block index (within the sequence) of the next step to load
-    int nxt_in = s_lo - tbl_base * steps_per_blk; // its step index inside that block
-
     // Row r of a K tile holds token 4 (r % 4) + r / 4 of the tile, so that result element
     // (tile t, quad element e) of lane group g is token 4 (4 t + e) + g of the step.
     const uint32_t k_lane = (uint32_t)((4 * (n & 3) + (n >> 2)) * a.tok_stride + 8 * g);
     const uint32_t v_lane = (uint32_t)(g * a.tok_stride + 8 * n);
     const uint32_t tile_off = (uint32_t)(16 * a.tok_stride);
     const uint32_t quad_off = (uint32_t)(4 * a.tok_stride);
+    const uint16_t* dummy = a.q;   // 256 readable bytes that stay in cache
 
-    u32x4 kreg[2][4];
+    u32x4 kbuf[2][2][4];
     u32x4 vreg[8];
 
-    // Issues the 16 loads of the next step in line and advances the (block, step-in-block) cursor.
-    auto issue_loads = [&]() {
-        if (nxt_bi - tbl_base >= 64) {   // only for segments longer than 64 blocks
-            tbl_base = nxt_bi;
-            tblv = (tbl_base + lane <= blk_last) ? btrow[tbl_base + lane] : 0;
+    auto issue_k = [&](auto PC) {
+        constexpr int P = decltype(PC)::value;
+        const uint16_t* kb = dummy;
+        uint32_t lane_off = 0, t_off = 0;
+        if (kcur.live()) {
+            kb = a.k + ((int64_t)block_id(kcur) * a.blk_stride + (int64_t)(kcur.in * kStep) * a.tok_stride + (int64_t)h * kD);
+            lane_off = k_lane;
+            t_off = tile_off;
+            kcur.advance(plan, steps_per_blk);
         }
-        int blk = __builtin_amdgcn_readlane(tblv, nxt_bi - tbl_base);
-        blk = blk < 0 ? 0 : (blk >= a.num_blocks ? a.num_blocks - 1 : blk);
-        const int64_t base = (int64_t)blk * a.blk_stride + (int64_t)(nxt_in * kStep) * a.tok_stride + (int64_t)h * kD;
-        const uint16_t* kb = a.k + base;
-        const uint16_t* vb = a.v + base;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) kreg[t][j] = load16(kb + (t * tile_off + k_lane) + 32 * j);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) vreg[i] = load16(vb + (i * quad_off + v_lane));
-        if (++nxt_in == steps_per_blk) {
-            nxt_in = 0;
-            ++nxt_bi;
+            for (int j = 0; j < 4; ++j) kbuf[P][t][j] = load16(kb + (t * t_off + lane_off) + 32 * j);
+    };
+    auto issue_v = [&]() {
+        const uint16_t* vb = dummy;
+        uint32_t lane_off = 0, q_off = 0;
+        if (vcur.live()) {
+            vb = a.v + ((int64_t)block_id(vcur) * a.blk_stride + (int64_t)(vcur.in * kStep) * a.tok_stride + (int64_t)h * kD);
+            lane_off = v_lane;
+            q_off = quad_off;
+            vcur.advance(plan, steps_per_blk);
         }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) vreg[i] = load16(vb + (i * q_off + lane_off));
     };
 
-    issue_loads();
+    // Leaves the partial result of the segment just finished and resets the accumulators.
+    auto flush = [&](int b) {
+        float l_tot = l_run + __shfl_xor(l_run, 16);
+        l_tot += __shfl_xor(l_tot, 32);
+        const int64_t slot = (int64_t)h * a.slots_per_head + w + b;
+        if (n < G) {
+            float* po = a.po + (slot * G + n) * kD + 4 * g;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) *reinterpret_cast<f32x4*>(po + 16 * t) = acc[t];
+            if (g == 0) *reinterpret_cast<float2*>(a.ml + (slot * G + n) * 2) = make_float2(m_run, l_tot);
+        }
+#pragma unroll
+        for (int t = 0; t < 8; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        m_run = -INFINITY;
+        l_run = 0.f;
+    };
 
-    for (int s = s_lo; s < s_hi; ++s) {
+    auto step = [&](auto PC) {
+        constexpr int P = decltype(PC)::value;
         // ---- S^T = K Q^T
         f32x4 sc[2];
 #pragma unroll
@@ -168,27 +266,14 @@ __device__ __forceinline__ void run_segment(const DecodeArgs& a, unsigned char* 
             sc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kreg[t][j]), qreg[j], sc[t], 0, 0, 0);
+                sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kbuf[P][t][j]), as_bf16x8(qreg[j]), sc[t], 0, 0, 0);
         }
-
-        // ---- stage V (rows past the end of the sequence are zeroed: their P is 0 and 0 * NaN must not leak)
-        const int tok0 = s * kStep;
-        const bool tail = tok0 + kStep > len;
-        if (tail) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                if (tok0 + 4 * i + g >= len) vreg[i] = u32x4{0u, 0u, 0u, 0u};
-        }
-        lds_order();
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-            *reinterpret_cast<u32x4*>(lds + (4 * i + g) * kLdsRow + n * 16) = vreg[i];
-        lds_order();
-
-        // ---- prefetch the next step while this one is being reduced
-        if (s + 1 < s_hi) issue_loads();
+        issue_k(PC);   // refill this K buffer with the step after next
 
         // ---- online softmax, base 2
+        const int len = cseg.len;
+        const int tok0 = ccur.s * kStep;
+        const bool tail = tok0 + kStep > len;
         float sv[8];
 #pragma unroll
         for (int t = 0; t < 2; ++t)
@@ -218,11 +303,24 @@ __device__ __forceinline__ void run_segment(const DecodeArgs& a, unsigned char* 
         bf16x8 pb;
 #pragma unroll
         for (int i = 0; i < 8; ++i) pb[i] = (__bf16)pv[i];
+
+        // ---- stage V (rows past the end of the sequence are zeroed: their P is 0 and 0 * NaN must not leak)
+        if (tail) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (tok0 + 4 * i + g >= len) vreg[i] = u32x4{0u, 0u, 0u, 0u};
+        }
+        lds_order();
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            *reinterpret_cast<u32x4*>(lds + (4 * i + g) * kLdsRow + n * 16) = vreg[i];
+        lds_order();
+        issue_v();     // V of the next step
+
         if (__any(alpha != 1.f)) {
 #pragma unroll
             for (int t = 0; t < 8; ++t) acc[t] *= alpha;
         }
-
         // ---- O^T += V^T P^T : A operand element i of lane (g, n) is V[token 4 i + g][16 t + n]
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
@@ -237,21 +335,33 @@ __device__ __forceinline__ void run_segment(const DecodeArgs& a, unsigned char* 
             acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vt), pb, acc[t], 0, 0, 0);
         }
         lds_order();
-    }
 
-    // ---- leave the partial result of this segment
-    l_run += __shfl_xor(l_run, 16);
-    l_run += __shfl_xor(l_run, 32);
-    const int64_t slot = (int64_t)h * a.slots_per_head + w + b;
-    if (n < G) {
-        float* po = a.po + (slot * G + n) * kD + 4 * g;
+        // ---- next step; at a sequence boundary leave the partial result and switch Q
+        const int seg_before = ccur.seg;
+        ccur.advance(plan, steps_per_blk);
+        if (ccur.seg != seg_before) {
+            flush(cseg.b);
+            if (ccur.live()) {
+                cseg = read_rec(plan, ccur.seg);
 #pragma unroll
-        for (int t = 0; t < 8; ++t) *reinterpret_cast<f32x4*>(po + 16 * t) = acc[t];
-        if (g == 0) {
-            float2 v2 = make_float2(m_run, l_run);
-            *reinterpret_cast<float2*>(a.ml + (slot * G + n) * 2) = v2;
+                for (int j = 0; j < 4; ++j) qreg[j] = qnext[j];
+                if (ccur.seg + 1 < nseg)
+                    load_q(__builtin_amdgcn_readfirstlane(plan[(ccur.seg + 1) * kPlanInts]), qnext);
+            }
         }
+    };
+
+    using P0 = std::integral_constant<int, 0>;
+    using P1 = std::integral_constant<int, 1>;
+    issue_k(P0{});
+    issue_v();
+    issue_k(P1{});
+    int i = 0;
+    for (; i + 1 < total_steps; i += 2) {
+        step(P0{});
+        step(P1{});
     }
+    if (i < total_steps) step(P0{});
 }
 
 __global__ void __launch_bounds__(512) paged_decode_split_kernel(DecodeArgs a) {
@@ -262,30 +372,41 @@ __global__ void __launch_bounds__(512) paged_decode_split_kernel(DecodeArgs a) {
     const int h = __builtin_amdgcn_readfirstlane(blockIdx.y * waves + wave);
     const int w = blockIdx.x;
     const int W = gridDim.x;
-    unsigned char* lds = lds_all + wave * kLdsWave;
+    unsigned char* lds = lds_all + wave * kLdsPerWave;
+    int* plan = reinterpret_cast<int*>(lds + kLdsWave);
+    const int steps_per_blk = a.block_size / kStep;
 
-    // total number of steps
-    int total = 0;
-    for (int c = 0; c < a.batch; c += 64) {
+    // total number of steps (the first 64 lengths stay in registers for the second pass)
+    const int len0 = lane < a.batch ? a.ctx[lane] : 0;
+    int total = wave_sum(steps_of(len0));
+    for (int c = 64; c < a.batch; c += 64) {
         const int i = c + lane;
         total += wave_sum(i < a.batch ? steps_of(a.ctx[i]) : 0);
     }
     total = __builtin_amdgcn_readfirstlane(total);   // wave-uniform: keep the plan in scalar registers
-    int span = (total + W - 1) / W;
-    span = span < kMinSpan ? kMinSpan : span;
+
+    // Equal shares: the first `rem` workgroups take one step more.  Tiny problems use fixed spans of
+    // kMinSpan steps instead, so the number of partial results stays small.
+    int lo, hi;
+    if (total >= W * kMinSpan) {
+        const int q = total / W, rem = total - q * W;
+        lo = w * q + (w < rem ? w : rem);
+        hi = lo + q + (w < rem ? 1 : 0);
+    } else {
+        lo = w * kMinSpan;
+        hi = lo + kMinSpan < total ? lo + kMinSpan : total;
+    }
     if (w == 0 && h == 0 && lane == 0) {
         a.header[0] = W;
-        a.header[1] = span;
-        a.header[2] = total;
+        a.header[1] = total;
     }
-    const int lo = w * span;
-    const int hi = (lo + span < total) ? lo + span : total;
     if (lo >= hi) return;
 
+    int nseg = 0, nord = 0, nsteps = 0, tblv = 0;
     int running = 0;
     for (int c = 0; c < a.batch; c += 64) {
         const int i = c + lane;
-        const int len = i < a.batch ? a.ctx[i] : 0;
+        const int len = c == 0 ? len0 : (i < a.batch ? a.ctx[i] : 0);
         const int cnt = steps_of(len);
         const int incl = wave_inclusive_scan(cnt, lane);
         const int start = running + incl - cnt;
@@ -304,10 +425,33 @@ __global__ void __launch_bounds__(512) paged_decode_split_kernel(DecodeArgs a) {
                 if (s_lo == 0) a.seg_first[b] = w;
                 if (s_hi == en - st) a.seg_last[b] = w;
             }
-            run_segment(a, lds, b, ln, s_lo, s_hi, h, w, lane);
+            const int blk0 = s_lo / steps_per_blk;
+            const int nblk = (s_hi - 1) / steps_per_blk - blk0 + 1;
+            if (nseg == kMaxSegs || (nseg > 0 && nord + nblk > 64)) {
+                lds_order();
+                run_batch(a, lds, plan, nseg, nsteps, tblv, h, w, lane);
+                lds_order();
+                nseg = nord = nsteps = 0;
+                tblv = 0;
+            }
+            if (lane == 0) {
+                int* p = plan + nseg * kPlanInts;
+                p[0] = b; p[1] = ln; p[2] = s_lo; p[3] = s_hi; p[4] = nord; p[5] = s_lo - blk0 * steps_per_blk; p[6] = blk0;
+            }
+            {   // gather this segment's block ids into lanes [nord, nord + nblk)
+                const int k = lane - nord;
+                if (k >= 0 && k < nblk && lane < 64) tblv = a.bt[(int64_t)b * a.bt_stride0 + blk0 + k];
+            }
+            ++nseg;
+            nord += nblk;
+            nsteps += s_hi - s_lo;
         }
         running += __builtin_amdgcn_readlane(incl, 63);
         if (running >= hi) break;
+    }
+    if (nseg > 0) {
+        lds_order();
+        run_batch(a, lds, plan, nseg, nsteps, tblv, h, w, lane);
     }
 }
 
@@ -324,34 +468,49 @@ struct MergeArgs {
     int batch;
 };
 
-// grid (batch, Hkv), 128 threads: thread d folds the segments of (sequence, KV head) for every
-// query head of the group.
-__global__ void __launch_bounds__(128) paged_decode_merge_kernel(MergeArgs a) {
+// grid (batch, Hkv), 256 threads: each thread folds the segments of one (query head, 4 output
+// columns) item of its (sequence, KV head) with the running (max, sum) rule, loads of four
+// segments in flight at a time.
+__global__ void __launch_bounds__(256) paged_decode_merge_kernel(MergeArgs a) {
     const int b = blockIdx.x;
     const int h = blockIdx.y;
-    const int d = threadIdx.x;
     const int G = a.group;
-    uint16_t* orow = a.out + (int64_t)b * a.out_stride0 + (int64_t)h * G * kD + d;
-    if (a.ctx[b] <= 0) {
-        for (int n = 0; n < G; ++n) orow[n * kD] = 0;
-        return;
-    }
+    const bool empty = a.ctx[b] <= 0;
     const int W = a.header[0];
-    const int w0 = a.seg_first[b];
-    const int w1 = a.seg_last[b];
+    const int w0 = empty ? 0 : a.seg_first[b];
+    const int w1 = empty ? -1 : a.seg_last[b];
     const int64_t slot0 = (int64_t)h * (W + a.batch) + b;
-    for (int n = 0; n < G; ++n) {
-        float mx = -INFINITY;
-        for (int w = w0; w <= w1; ++w) mx = fmaxf(mx, a.ml[((slot0 + w) * G + n) * 2]);
-        float num = 0.f, den = 0.f;
-        for (int w = w0; w <= w1; ++w) {
-            const float* mlp = a.ml + ((slot0 + w) * G + n) * 2;
-            const float wt = __builtin_amdgcn_exp2f(mlp[0] - mx);
-            den += wt * mlp[1];
-            num += wt * a.po[((slot0 + w) * G + n) * kD + d];
+    for (int item = threadIdx.x; item < G * 32; item += 256) {
+        const int n = item >> 5, c4 = item & 31;
+        float m = -INFINITY, den = 0.f;
+        f32x4 num = {0.f, 0.f, 0.f, 0.f};
+        for (int wb = w0; wb <= w1; wb += 4) {
+            float2 mlv[4];
+            f32x4 pov[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int wu = wb + u <= w1 ? wb + u : w1;
+                const int64_t row = (slot0 + wu) * G + n;
+                mlv[u] = *reinterpret_cast<const float2*>(a.ml + row * 2);
+                pov[u] = *reinterpret_cast<const f32x4*>(a.po + row * kD + 4 * c4);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (wb + u > w1) break;
+                const float m_new = fmaxf(m, mlv[u].x);
+                const float f_old = __builtin_amdgcn_exp2f(m - m_new);
+                const float f_new = __builtin_amdgcn_exp2f(mlv[u].x - m_new);
+                den = den * f_old + mlv[u].y * f_new;
+                num = num * f_old + pov[u] * f_new;
+                m = m_new;
+            }
         }
-        const __bf16 r = (__bf16)(num / den);
-        orow[n * kD] = __builtin_bit_cast(uint16_t, r);
+        const float inv = den > 0.f ? 1.f / den : 0.f;
+        union { __bf16 hv[4]; u32x2 u; } r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r.hv[e] = (__bf16)(num[e] * inv);
+        uint16_t* op = a.out + (int64_t)b * a.out_stride0 + (int64_t)(h * G + n) * kD + 4 * c4;
+        *reinterpret_cast<u32x2*>(op) = r.u;
     }
 }
 
@@ -466,11 +625,11 @@ int infer_paged_decode_split_bf16(const void* q, int64_t q_stride0, const void* 
     a.po = (float*)(base + ws.po_off);
     a.slots_per_head = L.W + (int)batch;
 
-    const size_t lds_bytes = (size_t)L.waves * kLdsWave;
+    const size_t lds_bytes = (size_t)L.waves * kLdsPerWave;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)paged_decode_split_kernel,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 8 * kLdsWave);
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 8 * kLdsPerWave);
         if (e != hipSuccess) return (int)e;
         attr_set = true;
     }
@@ -502,7 +661,7 @@ int infer_paged_decode_merge_bf16(void* out, int64_t out_stride0, const int32_t*
     m.ml = (const float*)(base + ws.ml_off);
     m.po = (const float*)(base + ws.po_off);
     m.batch = (int)batch;
-    dim3 grid((unsigned)batch, (unsigned)num_kv_heads, 1), block(128, 1, 1);
+    dim3 grid((unsigned)batch, (unsigned)num_kv_heads, 1), block(256, 1, 1);
     hipLaunchKernelGGL(paged_decode_merge_kernel, grid, block, 0, (hipStream_t)stream, m);
     return (int)hipGetLastError();
 }
