@@ -1,0 +1,62 @@
+"""The C-ABI library loads without a GPU and exports every symbol include/infer_kv.h declares."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from infer_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    names = []
+    for fn in sorted(os.listdir(os.path.join(ROOT, "include"))):
+        if fn.endswith(".h"):
+            text = open(os.path.join(ROOT, "include", fn)).read()
+            text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+            names += re.findall(r"\b(infer_[a-z0-9_]+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_functions()
+    for must in ("infer_kv_append_bf16", "infer_paged_decode_bf16", "infer_paged_decode_workspace_bytes"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol_and_binding_covers_it():
+    lib = _lib.load()
+    for name in declared_functions():
+        assert hasattr(lib, name), f"{name} declared in include/ but not exported"
+        assert name in _lib.SIGNATURES, f"{name} has no ctypes signature"
+    for name in _lib.SIGNATURES:
+        assert name in declared_functions(), f"{name} bound but not declared in include/"
+
+
+def test_host_only_entry_points():
+    lib = _lib.load()
+    assert lib.infer_kv_version() == b"0.1"
+    assert b"workspace" in lib.infer_kv_strerror(-3)
+    assert lib.infer_paged_decode_workspace_bytes(64, 32, 8, 128) > 0
+    assert lib.infer_paged_decode_workspace_bytes(64, 32, 8, 64) == 0        # head_dim not built
+    assert lib.infer_paged_decode_workspace_bytes(64, 30, 8, 128) == 0       # Hq % Hkv != 0
+    small = lib.infer_paged_decode_workspace_bytes(1, 32, 8, 128)
+    assert lib.infer_paged_decode_workspace_bytes(512, 32, 8, 128) > small
+
+
+def test_argument_errors_are_reported_before_anything_is_launched():
+    lib = _lib.load()
+    # null pointers / bad sizes are rejected by the host-side checks (no device is touched)
+    assert lib.infer_kv_append_bf16(None, 1024, None, 1024, None, None, None, 4, 1024, 256, None) == -1
+    assert lib.infer_kv_append_bf16(None, 1024, None, 1024, None, None, None, 0, 1024, 256, None) == 0
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.addressof(buf)
+    p16 = (p + 15) & ~15
+    assert lib.infer_kv_append_bf16(p16, 1024, p16, 1024, p16, p16, p16, 4, 1020, 256, None) == -2   # dkv % 8
+    assert lib.infer_kv_append_bf16(p16 + 2, 1024, p16, 1024, p16, p16, p16, 4, 1024, 256, None) == -2
+    assert lib.infer_paged_decode_bf16(None, 0, None, None, 0, 0, None, 0, None, 0, None,
+                                       1, 32, 8, 128, 256, 4, 1.0, None, 0, None) == -1
+    with pytest.raises(RuntimeError, match="workspace too small"):
+        _lib.check(-3, "x")
