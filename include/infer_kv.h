@@ -34,6 +34,9 @@ extern "C" {
 #define INFER_KV_EALIGN       -2   /* pointer or stride not aligned for the vector path         */
 #define INFER_KV_EWORKSPACE   -3   /* workspace too small                                       */
 #define INFER_KV_EUNSUPPORTED -4   /* head_dim / group size / block size outside what is built  */
+#define INFER_KV_ESTATE       -5   /* block pool: the call violates an invariant the reference
+                                      asserts (double allocate, out of blocks, ...); see
+                                      infer_pool_last_error()                                   */
 
 /* Library version, "major.minor". */
 const char* infer_kv_version(void);
@@ -128,6 +131,51 @@ int infer_paged_decode_merge_bf16(void* out, int64_t out_stride0,
 /* Tuning knob: number of workgroups along the KV-split axis used by the decode kernels
  * (0 = choose from the device's CU count).  Process-wide; returns the previous value. */
 int infer_paged_decode_set_split_workgroups(int workgroups);
+
+/* ------------------------------------------------------------------ 3. block pool (host only)
+ * C view of infer::BlockPool (include/infer_kv/block_pool.hpp), the native counterpart of the
+ * reference's Python BlockManager (infer/engine/block_mannager.py:44-133), which is the block
+ * pool the reference engine runs (its C++ include/kvcache.hpp / src/kvcache.cc is never
+ * compiled).  Token ids are int64, block ids int32.  Functions that the reference guards with
+ * `assert` return INFER_KV_ESTATE and leave a message in infer_pool_last_error() (thread local).
+ */
+typedef struct infer_pool infer_pool;
+
+infer_pool* infer_pool_create(int32_t num_blocks, int32_t block_size);   /* BlockManager.__init__ :46-52 */
+void infer_pool_destroy(infer_pool* pool);
+const char* infer_pool_last_error(void);
+int32_t infer_pool_num_free(const infer_pool* pool);
+int32_t infer_pool_num_used(const infer_pool* pool);
+
+/* can_allocate :76-77 -> 1 / 0. */
+int infer_pool_can_allocate(const infer_pool* pool, int64_t num_tokens);
+
+/* allocate :79-103.  Writes ceil(num_tokens / block_size) block ids to table_out and returns the
+ * number of tokens already present in the cache (a multiple of block_size), or a negative code. */
+int64_t infer_pool_allocate(infer_pool* pool, const int64_t* token_ids, int64_t num_tokens,
+                            int32_t* table_out, int64_t table_capacity);
+
+/* deallocate :105-112 (references dropped in reverse table order). */
+int infer_pool_deallocate(infer_pool* pool, const int32_t* table, int64_t num_blocks);
+
+/* can_append :114-115 -> 1 / 0. */
+int infer_pool_can_append(const infer_pool* pool, int64_t seq_len);
+
+/* may_append :117-133, called after the sequence grew to seq_len tokens.  May append one block id
+ * to `table` (capacity must allow num_blocks + 1 then).  Returns the new number of blocks. */
+int64_t infer_pool_may_append(infer_pool* pool, const int64_t* token_ids, int64_t seq_len,
+                              int32_t* table, int64_t num_blocks, int64_t table_capacity);
+
+/* compute_hash :54-60: xxh64(seed 0) over [prefix hash as 8 LE bytes, if has_prefix] ++ int64 LE ids. */
+uint64_t infer_pool_hash(const int64_t* token_ids, int64_t n, int has_prefix, uint64_t prefix_hash);
+
+/* XXH64 itself (the reference gets it from the un-vendored pip package `xxhash`). */
+uint64_t infer_xxh64(const void* data, size_t len, uint64_t seed);
+
+/* Introspection. */
+int32_t infer_pool_ref_count(const infer_pool* pool, int32_t block_id);
+int infer_pool_block_hash(const infer_pool* pool, int32_t block_id, uint64_t* hash_out);  /* 1 if sealed */
+int64_t infer_pool_free_ids(const infer_pool* pool, int32_t* out, int64_t capacity);      /* FIFO order */
 
 #ifdef __cplusplus
 }

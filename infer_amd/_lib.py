@@ -31,6 +31,21 @@ SIGNATURES = {
                                                  _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp, _sz, _vp]),
     "infer_paged_decode_merge_bf16": (_c.c_int, [_vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _sz, _vp]),
     "infer_paged_decode_set_split_workgroups": (_c.c_int, [_c.c_int]),
+    "infer_pool_create": (_vp, [_i32, _i32]),
+    "infer_pool_destroy": (None, [_vp]),
+    "infer_pool_last_error": (_c.c_char_p, []),
+    "infer_pool_num_free": (_i32, [_vp]),
+    "infer_pool_num_used": (_i32, [_vp]),
+    "infer_pool_can_allocate": (_c.c_int, [_vp, _i64]),
+    "infer_pool_allocate": (_i64, [_vp, _vp, _i64, _vp, _i64]),
+    "infer_pool_deallocate": (_c.c_int, [_vp, _vp, _i64]),
+    "infer_pool_can_append": (_c.c_int, [_vp, _i64]),
+    "infer_pool_may_append": (_i64, [_vp, _vp, _i64, _vp, _i64, _i64]),
+    "infer_pool_hash": (_c.c_uint64, [_vp, _i64, _c.c_int, _c.c_uint64]),
+    "infer_xxh64": (_c.c_uint64, [_vp, _sz, _c.c_uint64]),
+    "infer_pool_ref_count": (_i32, [_vp, _i32]),
+    "infer_pool_block_hash": (_c.c_int, [_vp, _i32, _vp]),
+    "infer_pool_free_ids": (_i64, [_vp, _vp, _i64]),
 }
 
 
