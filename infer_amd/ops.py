@@ -142,5 +142,14 @@ def flash_attn_decode(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, is_caus
     paged_attn_decode(Q, K, V, block_table, context_lens, softmax_scale, O)
 
 
+def flash_attn_varlen_func(q, k, v, *, max_seqlen_q, cu_seqlens_q, max_seqlen_k, cu_seqlens_k,
+                           softmax_scale=None, causal=True, block_table=None):
+    """Packed variable-length causal attention (keyword set of ``infer/ops/attention.py:113-116``).
+
+    Not built yet: this tree implements the decode half of the path first.  Raises instead of
+    silently computing something else."""
+    raise NotImplementedError("flash_attn_varlen_func: the paged varlen prefill kernel is not built in this version")
+
+
 def set_split_workgroups(n: int) -> int:
     return _lib.load().infer_paged_decode_set_split_workgroups(int(n))
