@@ -21,6 +21,12 @@ import torch
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per launch of the decode split kernel on this workload, from two rocprofv3 --pmc passes
+# of `python3 bench.py --counters` (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000 KiB; the factors are what
+# the same counters read for the 1 GiB plain copy run first): 631,008 KiB read + 5,057 KiB written.
+# Summary under profiles/decode_cfg2_hbm_counters.txt.  The workload is seeded, so the figure is stable.
+MEASURED_TRAFFIC_BYTES = (631008 + 5057) * 1024
+
 
 def gpu_time_ms(fn, iters, warmup):
     """Average milliseconds per call of ``fn`` over ``iters`` calls, HIP events on the current stream."""
@@ -72,6 +78,9 @@ def main():
     ap.add_argument("--copies", type=int, default=4, help="independent cache copies walked round-robin")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--splits", type=int, default=0, help="KV-split workgroups (0 = library default)")
+    ap.add_argument("--counters", action="store_true",
+                    help="short untimed run for `rocprofv3 --pmc`: a 1 GiB plain copy (x3), the decode op (x5), "
+                         "a prefill-sized append (x3)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this path needs no collective and every box here has one GPU; "
@@ -87,6 +96,23 @@ def main():
         ops.set_split_workgroups(args.splits)
     wl = workloads.cfg2(device=dev)
     b, hq, hkv, d = len(wl.lengths), wl.num_q_heads, wl.num_kv_heads, wl.head_dim
+    if args.counters:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        out = torch.empty((b, hq, d), dtype=torch.bfloat16, device=dev)
+        ws = ops.decode_workspace(dev, b, hq, hkv, d)
+        p3 = workloads.cfg3(device=dev)
+        torch.cuda.synchronize()
+        for _ in range(3):
+            dst.copy_(src)      # plain copy of known size: 1 GiB read, 1 GiB written
+        for _ in range(5):
+            ops.paged_attn_decode(wl.q, wl.k_cache, wl.v_cache, wl.block_table, wl.context_lens, wl.scale, out, ws)
+        for _ in range(3):
+            ops.store_kvcache(p3.k_new, p3.v_new, p3.k_cache, p3.v_cache, p3.slot_mapping)
+        torch.cuda.synchronize()
+        print(json.dumps({"counters_run": True, "copy_bytes": 1 << 30, "decode_algorithmic_bytes": wl.decode_bytes,
+                          "append_algorithmic_bytes": p3.append_bytes}))
+        return
     k_copies = [wl.k_cache] + [torch.randn_like(wl.k_cache) for _ in range(args.copies - 1)]
     v_copies = [wl.v_cache] + [torch.randn_like(wl.v_cache) for _ in range(args.copies - 1)]
     out = torch.empty((b, hq, d), dtype=torch.bfloat16, device=dev)
@@ -151,7 +177,7 @@ def main():
         "wall_ms_per_step": round(wall_ms, 5),
         "roofline": {"bound": "hbm", "kernel": "paged_decode_split_kernel", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": None, "avg_kernel_ms": round(split_ms, 5)},
+                     "traffic": MEASURED_TRAFFIC_BYTES, "avg_kernel_ms": round(split_ms, 5)},
         "append": {"decode_rows": b, "decode_us": round(ap_small_ms * 1e3, 2),
                    "prefill_rows": int(p3.slot_mapping.numel()), "prefill_bytes": p3.append_bytes,
                    "prefill_us": round(ap_ms * 1e3, 2), "prefill_GBps": round(append_gbs, 1),

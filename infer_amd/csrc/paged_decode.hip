@@ -13,7 +13,8 @@
 //   KV head, so a workgroup reads whole 2 KiB token rows while each wavefront runs its own
 //   private pipeline (no workgroup barrier anywhere).  A span may cover the tail of one
 //   sequence and the head of the next: each (sequence, span) piece is a "segment" and leaves a
-//   partial result; the merge kernel folds the segments of a sequence together.
+//   partial result (parked in LDS, stored once the wavefront has issued its last load); the merge
+//   kernel folds the segments of a sequence together.
 //
 // Per step and wavefront (KV head h, G = Hq/Hkv query heads):
 //   S^T[token, head] = K[token, :] . Q^T        2 tiles x 4 v_mfma_f32_16x16x32_bf16
@@ -104,7 +105,11 @@ __device__ __forceinline__ void lds_order() { __asm__ volatile("" ::: "memory");
 constexpr int kPlanInts = 8;        // ints per segment record
 constexpr int kMaxSegs = 32;        // segments per batch (a span with more is run in several batches)
 constexpr int kPlanBytes = kMaxSegs * kPlanInts * 4;
-constexpr int kLdsPerWave = kLdsWave + kPlanBytes;
+// Partial results of finished segments wait in LDS until the wavefront has issued its last load:
+// a global store in the middle of the stream would make the outstanding-load counter unordered
+// (loads and stores share it) and force a full drain of the prefetch pipeline.
+constexpr int kDeferBytes = 8448;   // 4 segments at group size 4, 2 at 8, 1 at 16
+constexpr int kLdsPerWave = kLdsWave + kPlanBytes + kDeferBytes;
 
 struct SegRec {      // one record of the plan, all wave-uniform
     int b;           // sequence
@@ -158,7 +163,12 @@ struct StepCursor {
 // batch are redirected to one dummy 16-byte location instead of being skipped, which keeps the
 // number of outstanding loads at every wait independent of control flow.
 __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* lds, const int* plan, int nseg,
-                                          int total_steps, int tblv, int h, int w, int lane) {
+                                          int total_steps, int tblv_loaded, int h, int w, int lane) {
+    // The block ids were gathered by vector loads.  Hand them to the loop as a plain register value:
+    // otherwise every later read of this register is treated as "may still be in flight" and gets a
+    // wait that also drains the K/V loads issued since, which defeats the pipeline.
+    int tblv;
+    __asm__ volatile("v_mov_b32 %0, %1" : "=v"(tblv) : "v"(tblv_loaded));
     const int g = lane >> 4;   // lane group: the k-slice of MFMA operands, the row-quad of results
     const int n = lane & 15;   // operand row / result column
     const int G = a.group;
@@ -240,46 +250,56 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
         for (int i = 0; i < 8; ++i) vreg[i] = load16(vb + (i * q_off + lane_off));
     };
 
-    // Leaves the partial result of the segment just finished and resets the accumulators.
-    auto flush = [&](int b) {
+    // Partial results: parked in LDS (lane-private layout, valid lanes only), written out by drain().
+    unsigned char* defer = lds + kLdsWave + kPlanBytes;
+    const int slot_bytes = 520 * G;                 // 4G lanes x 8 x 16 B accumulators + G x 8 B (max, sum)
+    const int defer_cap = kDeferBytes / slot_bytes; // >= 1 for G <= 16
+    int ndef = 0, first_def = 0;                    // parked segments are first_def .. first_def + ndef - 1
+    const int vlane = g * G + n;                    // index among the 4G lanes that hold real heads
+
+    auto drain = [&]() {
+        for (int k = 0; k < ndef; ++k) {
+            const int b = __builtin_amdgcn_readfirstlane(plan[(first_def + k) * kPlanInts]);
+            const int64_t slot = (int64_t)h * a.slots_per_head + w + b;
+            const unsigned char* src = defer + k * slot_bytes;
+            if (n < G) {
+                float* po = a.po + (slot * G + n) * kD + 4 * g;
+#pragma unroll
+                for (int t = 0; t < 8; ++t)
+                    *reinterpret_cast<f32x4*>(po + 16 * t) = *reinterpret_cast<const f32x4*>(src + (vlane * 8 + t) * 16);
+                if (g == 0)
+                    *reinterpret_cast<float2*>(a.ml + (slot * G + n) * 2) =
+                        *reinterpret_cast<const float2*>(src + 512 * G + n * 8);
+            }
+        }
+        first_def += ndef;
+        ndef = 0;
+    };
+
+    // Parks the partial result of the segment just finished and resets the accumulators.
+    auto flush = [&]() {
         float l_tot = l_run + __shfl_xor(l_run, 16);
         l_tot += __shfl_xor(l_tot, 32);
-        const int64_t slot = (int64_t)h * a.slots_per_head + w + b;
-        if (n < G) {
-            float* po = a.po + (slot * G + n) * kD + 4 * g;
-#pragma unroll
-            for (int t = 0; t < 8; ++t) *reinterpret_cast<f32x4*>(po + 16 * t) = acc[t];
-            if (g == 0) *reinterpret_cast<float2*>(a.ml + (slot * G + n) * 2) = make_float2(m_run, l_tot);
+        if (ndef == defer_cap) {          // only when one span covers many short sequences
+            lds_order();
+            drain();
+            __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): leave no store in flight behind
         }
+        unsigned char* dst = defer + ndef * slot_bytes;
+        lds_order();
+        if (n < G) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) *reinterpret_cast<f32x4*>(dst + (vlane * 8 + t) * 16) = acc[t];
+            if (g == 0) *reinterpret_cast<float2*>(dst + 512 * G + n * 8) = make_float2(m_run, l_tot);
+        }
+        lds_order();
+        ++ndef;
 #pragma unroll
         for (int t = 0; t < 8; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
         m_run = -INFINITY;
         l_run = 0.f;
     };
 
-#if defined(INFER_KV_EXP) && INFER_KV_EXP >= 20
-    auto step = [&](auto PC) {
-        constexpr int P = decltype(PC)::value;
-        uint32_t x = 0;
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) x ^= kbuf[P][t][j].x ^ kbuf[P][t][j].y ^ kbuf[P][t][j].z ^ kbuf[P][t][j].w;
-        issue_k(PC);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) x ^= vreg[i].x ^ vreg[i].y ^ vreg[i].z ^ vreg[i].w;
-        issue_v();
-        acc[0][0] += __builtin_bit_cast(float, x);
-        const int seg_before = ccur.seg;
-        ccur.advance(plan, steps_per_blk);
-        if (ccur.seg != seg_before) {
-#if INFER_KV_EXP == 20
-            flush(cseg.b);
-#endif
-            if (ccur.live()) cseg = read_rec(plan, ccur.seg);
-        }
-    };
-#else
     auto step = [&](auto PC) {
         constexpr int P = decltype(PC)::value;
         // ---- S^T = K Q^T
@@ -363,7 +383,7 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
         const int seg_before = ccur.seg;
         ccur.advance(plan, steps_per_blk);
         if (ccur.seg != seg_before) {
-            flush(cseg.b);
+            flush();
             if (ccur.live()) {
                 cseg = read_rec(plan, ccur.seg);
 #pragma unroll
@@ -374,7 +394,6 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
         }
     };
 
-#endif
     using P0 = std::integral_constant<int, 0>;
     using P1 = std::integral_constant<int, 1>;
     issue_k(P0{});
@@ -386,6 +405,8 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
         step(P1{});
     }
     if (i < total_steps) step(P0{});
+    lds_order();
+    drain();
 }
 
 __global__ void __launch_bounds__(512) paged_decode_split_kernel(DecodeArgs a) {
@@ -425,44 +446,6 @@ __global__ void __launch_bounds__(512) paged_decode_split_kernel(DecodeArgs a) {
         a.header[1] = total;
     }
     if (lo >= hi) return;
-#if defined(INFER_KV_EXP) && INFER_KV_EXP == 30
-    {   // streaming probe inside the real launch: contiguous addressing, K double / V single buffered
-        const int g = lane >> 4, n = lane & 15;
-        const size_t per = total / W;
-        const size_t s0 = per * w;
-        const uint32_t tok = (uint32_t)a.tok_stride;
-        const uint32_t k_lane = (4 * (n & 3) + (n >> 2)) * tok + 8 * g;
-        const uint32_t v_lane = g * tok + 8 * n;
-        const uint16_t* kb = a.k + s0 * 32 * tok + h * 128;
-        const uint16_t* vb = a.v + s0 * 32 * tok + h * 128;
-        uint32_t accx = 0;
-        auto ldk = [&](u32x4 (&r)[8], size_t s) {
-            const uint16_t* p = kb + s * 32 * tok;
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) r[t*4+j] = *(const u32x4*)(p + t*16*tok + k_lane + 32*j);
-        };
-        auto ldv = [&](u32x4 (&r)[8], size_t s) {
-            const uint16_t* p = vb + s * 32 * tok;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) r[i] = *(const u32x4*)(p + i*4*tok + v_lane);
-        };
-        auto use = [&](u32x4 (&r)[8]) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) accx ^= r[i].x ^ r[i].y ^ r[i].z ^ r[i].w;
-        };
-        u32x4 k0[8], k1[8], vv[8];
-        ldk(k0, 0); ldv(vv, 0); ldk(k1, 1);
-        for (size_t s = 0; s + 3 < per; s += 2) {
-            use(k0); ldk(k0, s + 2); use(vv); ldv(vv, s + 1);
-            use(k1); ldk(k1, s + 3); use(vv); ldv(vv, s + 2);
-        }
-        use(k0); use(k1); use(vv);
-        if (accx == 0x12345678) a.header[5] = accx;
-        return;
-    }
-#endif
 
     int nseg = 0, nord = 0, nsteps = 0, tblv = 0;
     int running = 0;
