@@ -128,6 +128,33 @@ int infer_paged_decode_merge_bf16(void* out, int64_t out_stride0,
                                   const void* workspace, size_t workspace_bytes,
                                   void* stream);
 
+/* ------------------------------------------------------------------ 2b. paged varlen prefill attention
+ * Replaces flash_attn_varlen_func(Q, K, V, max_seqlen_q, cu_seqlens_q, max_seqlen_k, cu_seqlens_k,
+ * softmax_scale, causal=True, block_table) at infer/ops/attention.py:110-116.
+ *
+ * Queries are packed: q [total_q, Hq, D] (row stride q_stride0), sequence s owns rows
+ * [cu_seqlens_q[s], cu_seqlens_q[s+1]); out has the same layout.  Keys/values:
+ *   block_table != NULL : k, v are the paged caches [num_blocks, block_size, Hkv, D] and sequence s
+ *                         uses tokens [0, sk_s) of row s of the table, sk_s from cu_seqlens_k
+ *                         (the reference's prefix-cache case, attention.py:111-112);
+ *   block_table == NULL : k, v are packed rows [kv_rows, Hkv, D] indexed by cu_seqlens_k
+ *                         (kv_token_stride is the row stride, kv_block_stride is ignored).
+ * kv_rows = number of token rows addressable through k/v (packed: rows of the tensor; paged:
+ * num_blocks * block_size); it only bounds reads.  causal != 0 applies the bottom-right aligned
+ * mask (key j visible to query i of the sequence iff j <= i + (sk - sq)).  Queries of a sequence
+ * with sk == 0 produce zeros.  Same shape limits as the decode entry points.  No workspace.
+ */
+int infer_paged_prefill_bf16(const void* q, int64_t q_stride0,
+                             const void* k, const void* v,
+                             int64_t kv_block_stride, int64_t kv_token_stride, int64_t kv_rows,
+                             void* out, int64_t out_stride0,
+                             const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                             const int32_t* block_table, int64_t bt_stride0,
+                             int64_t num_seqs, int64_t max_seqlen_q,
+                             int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                             int64_t block_size, int64_t num_blocks,
+                             float scale, int causal, void* stream);
+
 /* Tuning knob: number of workgroups along the KV-split axis used by the decode kernels
  * (0 = choose from the device's CU count).  Process-wide; returns the previous value. */
 int infer_paged_decode_set_split_workgroups(int workgroups);

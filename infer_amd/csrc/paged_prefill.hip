@@ -1,0 +1,272 @@
+// Paged variable-length causal prefill attention for gfx950 (MI355X), bf16 in / fp32 accumulate.
+//
+// Replaces flash_attn_varlen_func(Q, K, V, cu_seqlens_q/k, max_seqlen_q/k, softmax_scale,
+// causal=True, block_table=...) at infer/ops/attention.py:110-116 of the reference.  With a block
+// table (a prefix of the sequence is already cached) the keys of sequence b are tokens [0, sk_b)
+// of its paged cache; without one K and V are the packed new rows.  The causal mask is aligned to
+// the bottom-right corner: key j is visible to query i iff j <= i + (sk - sq).
+//
+// One wavefront owns 16 consecutive queries of one query head and walks the visible keys in steps
+// of 32, with the same arithmetic as the decode kernel, the 16 MFMA columns now being 16 queries
+// instead of the heads of a GQA group:
+//   S^T[key, query] = K[key, :] . Q^T       2 tiles x 4 v_mfma_f32_16x16x32_bf16
+//   online softmax in the accumulator layout (lane = query, 8 keys per lane)
+//   O^T[d, query]  += V^T[d, key] . P^T     8 MFMAs, V staged through a wave-private LDS tile
+// The G wavefronts of a workgroup are the G query heads that share one KV head and the same query
+// tile, so they read the same K/V rows at about the same time (cache hits).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/infer_kv.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kD = 128;
+constexpr int kStep = 32;        // keys per step
+constexpr int kQTile = 16;       // queries per wavefront
+constexpr int kLdsRow = 288;     // 256 + 32: four consecutive rows hit disjoint LDS banks
+constexpr int kLdsWave = kStep * kLdsRow;
+
+struct PrefillArgs {
+    const uint16_t* q;
+    int64_t q_stride0;
+    const uint16_t* k;
+    const uint16_t* v;
+    int64_t blk_stride;
+    int64_t tok_stride;
+    uint16_t* out;
+    int64_t out_stride0;
+    const int32_t* cu_q;
+    const int32_t* cu_k;
+    const int32_t* bt;      // nullptr: packed K/V
+    int64_t bt_stride0;
+    int group;
+    int block_size;
+    int num_blocks;
+    int64_t total_k_rows;   // packed mode: rows in k/v (for clamping the tail)
+    float scale_log2;
+    int causal;
+};
+
+__device__ __forceinline__ bf16x8 as_bf16x8(u32x4 x) { return __builtin_bit_cast(bf16x8, x); }
+__device__ __forceinline__ u32x4 load16(const uint16_t* p) { return *reinterpret_cast<const u32x4*>(p); }
+__device__ __forceinline__ void lds_order() { __asm__ volatile("" ::: "memory"); }
+
+__global__ void __launch_bounds__(1024) paged_prefill_kernel(PrefillArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_all[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int g = lane >> 4, n = lane & 15;
+    const int b = blockIdx.y;
+    const int kvh = blockIdx.z;
+    const int head = kvh * a.group + wave;
+    unsigned char* lds = lds_all + wave * kLdsWave;
+
+    const int q_beg = a.cu_q[b], q_end = a.cu_q[b + 1];
+    const int k_beg = a.cu_k[b], k_end = a.cu_k[b + 1];
+    const int sq = q_end - q_beg, sk = k_end - k_beg;
+    const int q0 = blockIdx.x * kQTile;
+    if (q0 >= sq || sk <= 0) {
+        // queries without any key produce zeros (only possible when sk == 0)
+        if (q0 + n < sq && sk <= 0) {
+            uint16_t* op = a.out + (int64_t)(q_beg + q0 + n) * a.out_stride0 + (int64_t)head * kD + 4 * g;
+            for (int t = 0; t < 8; ++t) *reinterpret_cast<u32x2*>(op + 16 * t) = u32x2{0u, 0u};
+        }
+        return;
+    }
+    const int shift = sk - sq;                       // bottom-right alignment
+    const int my_q = q0 + n;                         // this lane's query (may be past sq: padded column)
+    const int my_limit = a.causal ? (my_q + shift < sk - 1 ? my_q + shift : sk - 1) : sk - 1;   // last visible key
+    int tile_last = q0 + kQTile - 1 < sq - 1 ? q0 + kQTile - 1 : sq - 1;
+    const int key_end = a.causal ? (tile_last + shift + 1 < sk ? tile_last + shift + 1 : sk) : sk;   // keys [0, key_end)
+    const int nsteps = (key_end + kStep - 1) / kStep;
+
+    // Q as the B operand: lane (g, n) holds Q[query n][32 j + 8 g .. +8]
+    bf16x8 qreg[4];
+    {
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        const bool live = my_q < sq;
+        const uint16_t* qp = a.q + (int64_t)(q_beg + (live ? my_q : 0)) * a.q_stride0 + (int64_t)head * kD + 8 * g;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) qreg[j] = as_bf16x8(live ? load16(qp + 32 * j) : z);
+    }
+
+    f32x4 acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+
+    const int krow = 4 * (n & 3) + (n >> 2);   // row r of a K tile holds key 4 (r % 4) + r / 4 of the tile
+    u32x4 kreg[2][4];
+    u32x4 vreg[8];
+
+    auto issue_loads = [&](int s) {
+        const int tok0 = s * kStep;
+        if (a.bt) {
+            int blk = __builtin_amdgcn_readfirstlane(a.bt[(int64_t)b * a.bt_stride0 + tok0 / a.block_size]);
+            blk = blk < 0 ? 0 : (blk >= a.num_blocks ? a.num_blocks - 1 : blk);
+            const int64_t base = (int64_t)blk * a.blk_stride + (int64_t)(tok0 % a.block_size) * a.tok_stride + (int64_t)kvh * kD;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    kreg[t][j] = load16(a.k + base + (int64_t)(16 * t + krow) * a.tok_stride + 8 * g + 32 * j);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) vreg[i] = load16(a.v + base + (int64_t)(4 * i + g) * a.tok_stride + 8 * n);
+        } else {
+            const int64_t row0 = (int64_t)k_beg + tok0;
+            const int64_t last = a.total_k_rows - 1;
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                int64_t r = row0 + 16 * t + krow;
+                r = r > last ? last : r;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) kreg[t][j] = load16(a.k + r * a.tok_stride + (int64_t)kvh * kD + 8 * g + 32 * j);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                int64_t r = row0 + 4 * i + g;
+                r = r > last ? last : r;
+                vreg[i] = load16(a.v + r * a.tok_stride + (int64_t)kvh * kD + 8 * n);
+            }
+        }
+    };
+
+    issue_loads(0);
+    for (int s = 0; s < nsteps; ++s) {
+        f32x4 sc[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            sc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kreg[t][j]), qreg[j], sc[t], 0, 0, 0);
+        }
+        const int tok0 = s * kStep;
+        // rows past the end of the sequence may hold anything: zero them in V (0 * NaN must not leak)
+        if (tok0 + kStep > sk) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (tok0 + 4 * i + g >= sk) vreg[i] = u32x4{0u, 0u, 0u, 0u};
+        }
+        lds_order();
+#pragma unroll
+        for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(lds + (4 * i + g) * kLdsRow + n * 16) = vreg[i];
+        lds_order();
+        if (s + 1 < nsteps) issue_loads(s + 1);
+
+        float sv[8];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sv[4 * t + e] = sc[t][e] * a.scale_log2;
+        if (tok0 + kStep - 1 > my_limit) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (tok0 + 4 * i + g > my_limit) sv[i] = -INFINITY;
+        }
+        float mx = sv[0];
+#pragma unroll
+        for (int i = 1; i < 8; ++i) mx = fmaxf(mx, sv[i]);
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx);
+        // a query that has seen no key yet keeps m = -inf: use 0 as the reference point then
+        const float m_ref = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
+        m_run = m_new;
+        float psum = 0.f;
+        float pv[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            pv[i] = __builtin_amdgcn_exp2f(sv[i] - m_ref);
+            psum += pv[i];
+        }
+        l_run = l_run * alpha + psum;
+        bf16x8 pb;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) pb[i] = (__bf16)pv[i];
+        if (__any(alpha != 1.f)) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) acc[t] *= alpha;
+        }
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const unsigned char* col = lds + g * kLdsRow + (16 * t + n) * 2;
+            u32x4 vt;
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                uint32_t lo = *reinterpret_cast<const uint16_t*>(col + (8 * p) * kLdsRow);
+                uint32_t hi = *reinterpret_cast<const uint16_t*>(col + (8 * p + 4) * kLdsRow);
+                vt[p] = lo | (hi << 16);
+            }
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vt), pb, acc[t], 0, 0, 0);
+        }
+        lds_order();
+    }
+
+    l_run += __shfl_xor(l_run, 16);
+    l_run += __shfl_xor(l_run, 32);
+    if (my_q < sq) {
+        const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+        uint16_t* op = a.out + (int64_t)(q_beg + my_q) * a.out_stride0 + (int64_t)head * kD + 4 * g;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            union { __bf16 hv[4]; u32x2 u; } r;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r.hv[e] = (__bf16)(acc[t][e] * inv);
+            *reinterpret_cast<u32x2*>(op + 16 * t) = r.u;
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" int infer_paged_prefill_bf16(const void* q, int64_t q_stride0, const void* k, const void* v,
+                                        int64_t kv_block_stride, int64_t kv_token_stride, int64_t kv_rows,
+                                        void* out, int64_t out_stride0, const int32_t* cu_seqlens_q,
+                                        const int32_t* cu_seqlens_k, const int32_t* block_table, int64_t bt_stride0,
+                                        int64_t num_seqs, int64_t max_seqlen_q, int64_t num_q_heads,
+                                        int64_t num_kv_heads, int64_t head_dim, int64_t block_size,
+                                        int64_t num_blocks, float scale, int causal, void* stream) {
+    if (!q || !k || !v || !out || !cu_seqlens_q || !cu_seqlens_k) return INFER_KV_EINVAL;
+    if (num_seqs <= 0 || max_seqlen_q < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || kv_rows <= 0) return INFER_KV_EINVAL;
+    if (max_seqlen_q == 0) return INFER_KV_OK;
+    if (head_dim != kD) return INFER_KV_EUNSUPPORTED;
+    if (num_q_heads % num_kv_heads != 0 || num_q_heads / num_kv_heads > 16) return INFER_KV_EUNSUPPORTED;
+    if (block_table && (block_size <= 0 || block_size % kStep != 0 || num_blocks <= 0)) return INFER_KV_EUNSUPPORTED;
+    if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) return INFER_KV_EALIGN;
+    if ((q_stride0 | kv_token_stride | out_stride0) & 7) return INFER_KV_EALIGN;
+    if (block_table && (kv_block_stride & 7)) return INFER_KV_EALIGN;
+    if (kv_token_stride < num_kv_heads * kD || q_stride0 < num_q_heads * kD || out_stride0 < num_q_heads * kD) return INFER_KV_EINVAL;
+    if (num_seqs > 65535 || num_kv_heads > 65535) return INFER_KV_EINVAL;
+    const int G = (int)(num_q_heads / num_kv_heads);
+    PrefillArgs a;
+    a.q = (const uint16_t*)q; a.q_stride0 = q_stride0;
+    a.k = (const uint16_t*)k; a.v = (const uint16_t*)v;
+    a.blk_stride = kv_block_stride; a.tok_stride = kv_token_stride;
+    a.out = (uint16_t*)out; a.out_stride0 = out_stride0;
+    a.cu_q = cu_seqlens_q; a.cu_k = cu_seqlens_k;
+    a.bt = block_table; a.bt_stride0 = bt_stride0;
+    a.group = G; a.block_size = (int)block_size; a.num_blocks = (int)num_blocks;
+    a.total_k_rows = kv_rows;
+    a.scale_log2 = scale * 1.4426950408889634f;
+    a.causal = causal ? 1 : 0;
+    const size_t lds_bytes = (size_t)G * kLdsWave;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)paged_prefill_kernel,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 16 * kLdsWave);
+        if (e != hipSuccess) return (int)e;
+        attr_set = true;
+    }
+    dim3 grid((unsigned)((max_seqlen_q + kQTile - 1) / kQTile), (unsigned)num_seqs, (unsigned)num_kv_heads);
+    dim3 block(64 * G, 1, 1);
+    hipLaunchKernelGGL(paged_prefill_kernel, grid, block, lds_bytes, (hipStream_t)stream, a);
+    return (int)hipGetLastError();
+}

@@ -144,11 +144,45 @@ def flash_attn_decode(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, is_caus
 
 def flash_attn_varlen_func(q, k, v, *, max_seqlen_q, cu_seqlens_q, max_seqlen_k, cu_seqlens_k,
                            softmax_scale=None, causal=True, block_table=None):
-    """Packed variable-length causal attention (keyword set of ``infer/ops/attention.py:113-116``).
+    """Packed variable-length attention (keyword set of ``infer/ops/attention.py:113-116``).
 
-    Not built yet: this tree implements the decode half of the path first.  Raises instead of
-    silently computing something else."""
-    raise NotImplementedError("flash_attn_varlen_func: the paged varlen prefill kernel is not built in this version")
+    ``q`` is ``[total_q, Hq, D]``.  With ``block_table`` the keys come from the paged caches
+    ``k``/``v`` ``[nblk, bs, Hkv, D]`` (prefix-cache case); without it ``k``/``v`` are the packed rows
+    ``[total_k, Hkv, D]``.  Returns ``[total_q, Hq, D]``.  ``max_seqlen_k`` is accepted for
+    signature compatibility; the kernel reads the lengths from ``cu_seqlens_k``."""
+    assert q.dim() == 3 and q.dtype == torch.bfloat16 and k.dtype == torch.bfloat16 and v.dtype == torch.bfloat16
+    tq, hq, d = q.shape
+    assert q.stride(2) == 1 and q.stride(1) == d
+    assert cu_seqlens_q.dtype == torch.int32 and cu_seqlens_k.dtype == torch.int32
+    assert cu_seqlens_q.is_contiguous() and cu_seqlens_k.is_contiguous()
+    nseq = cu_seqlens_q.numel() - 1
+    assert cu_seqlens_k.numel() == nseq + 1
+    _require_gpu(q, k, v, cu_seqlens_q, cu_seqlens_k)
+    if softmax_scale is None:
+        softmax_scale = d ** -0.5
+    out = torch.empty((tq, hq, d), dtype=q.dtype, device=q.device)
+    if tq == 0 or nseq == 0:
+        return out
+    if block_table is not None:
+        assert k.dim() == 4 and k.shape == v.shape and k.stride() == v.stride()
+        nblk, bs, hkv, dk = k.shape
+        assert dk == d and k.stride(3) == 1 and k.stride(2) == d
+        assert block_table.dtype == torch.int32 and block_table.shape[0] == nseq and block_table.stride(1) == 1
+        _require_gpu(block_table)
+        blk_stride, tok_stride, rows = k.stride(0), k.stride(1), nblk * bs
+        bt_ptr, bt_stride = block_table.data_ptr(), block_table.stride(0)
+    else:
+        assert k.dim() == 3 and k.shape == v.shape and k.stride() == v.stride()
+        rows, hkv, dk = k.shape
+        assert dk == d and k.stride(2) == 1 and k.stride(1) == d
+        blk_stride, tok_stride, bs, nblk = 0, k.stride(0), 0, 0
+        bt_ptr, bt_stride = None, 0
+    rc = _lib.load().infer_paged_prefill_bf16(
+        q.data_ptr(), q.stride(0), k.data_ptr(), v.data_ptr(), blk_stride, tok_stride, rows,
+        out.data_ptr(), out.stride(0), cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), bt_ptr, bt_stride,
+        nseq, int(max_seqlen_q), hq, hkv, d, bs, nblk, float(softmax_scale), int(bool(causal)), _stream_ptr(q))
+    _lib.check(rc, "flash_attn_varlen_func")
+    return out
 
 
 def set_split_workgroups(n: int) -> int:

@@ -1,0 +1,136 @@
+"""Paged varlen causal prefill attention on the GPU against the fp32 CPU oracle
+(oracle/paged_ref.varlen_prefill_ref).  Bar: bf16 output, max abs error <= 2e-2."""
+import numpy as np
+import pytest
+import torch
+
+from infer_amd import ops, workloads
+from infer_amd.attention import Attention
+from infer_amd.context import reset_context, set_context
+from oracle import paged_ref
+from tests.helpers import ATTN_ATOL, bits, f32
+
+pytestmark = pytest.mark.gpu
+
+
+def run_paged(wl):
+    """Reference step order (infer/ops/attention.py:108-116): append, then attend over the cache."""
+    kc, vc = wl.k_cache.clone(), wl.v_cache.clone()
+    ops.store_kvcache(wl.k_new, wl.v_new, kc, vc, wl.slot_mapping)
+    out = ops.flash_attn_varlen_func(wl.q, kc, vc, max_seqlen_q=wl.max_seqlen_q, cu_seqlens_q=wl.cu_seqlens_q,
+                                     max_seqlen_k=wl.max_seqlen_k, cu_seqlens_k=wl.cu_seqlens_k,
+                                     softmax_scale=wl.scale, causal=True, block_table=wl.block_table)
+    torch.cuda.synchronize()
+    return out, kc, vc
+
+
+def oracle_paged(wl, kc, vc):
+    return paged_ref.varlen_prefill_ref(bits(wl.q), bits(kc), bits(vc), wl.cu_seqlens_q.cpu().numpy(),
+                                        wl.cu_seqlens_k.cpu().numpy(), wl.scale,
+                                        block_table=wl.block_table.cpu().numpy())
+
+
+def test_cfg3_prefix_cached_prefill(gpu):
+    wl = workloads.cfg3().to(gpu)
+    out, kc, vc = run_paged(wl)
+    want = oracle_paged(wl, kc, vc)
+    err = float(np.abs(f32(out) - want).max())
+    print("cfg3 prefill max abs err", err)
+    assert np.isfinite(f32(out)).all() and err <= ATTN_ATOL
+
+
+@pytest.mark.parametrize("hq,hkv", [(8, 8), (16, 8), (32, 8), (64, 8), (8, 2), (16, 1)])
+def test_small_shapes_with_and_without_prefix(gpu, hq, hkv):
+    wl = workloads.make_prefill_workload("p", [1, 15, 16, 17, 33, 300, 257, 600], [0, 0, 0, 0, 0, 256, 256, 512],
+                                         hq, hkv, seed=hq + hkv, pad_fraction=0.1).to(gpu)
+    out, kc, vc = run_paged(wl)
+    assert np.abs(f32(out) - oracle_paged(wl, kc, vc)).max() <= ATTN_ATOL
+
+
+@pytest.mark.parametrize("bs", [32, 64, 512])
+def test_block_sizes(gpu, bs):
+    wl = workloads.make_prefill_workload("p", [70, 200, 5], [bs if bs <= 64 else 0, 0, 0], 16, 8, bs=bs, seed=bs,
+                                         pad_fraction=0.0).to(gpu)
+    out, kc, vc = run_paged(wl)
+    assert np.abs(f32(out) - oracle_paged(wl, kc, vc)).max() <= ATTN_ATOL
+
+
+def test_packed_keys_without_block_table_equals_causal_sdpa(gpu):
+    """No prefix cached: K and V are the packed new rows and sq == sk, which reduces to
+    scaled_dot_product_attention(is_causal=True), the convention of the reference's own attention
+    test (test/op.py:278-283, atol 2e-2)."""
+    g = torch.Generator().manual_seed(5)
+    lens = [64, 1, 100, 513]
+    hq, hkv, d = 32, 8, 128
+    t = sum(lens)
+    q = torch.randn((t, hq, d), generator=g).to(torch.bfloat16).to(gpu)
+    k = torch.randn((t, hkv, d), generator=g).to(torch.bfloat16).to(gpu)
+    v = torch.randn((t, hkv, d), generator=g).to(torch.bfloat16).to(gpu)
+    cu = torch.tensor(np.cumsum([0] + lens), dtype=torch.int32, device=gpu)
+    out = ops.flash_attn_varlen_func(q, k, v, max_seqlen_q=max(lens), cu_seqlens_q=cu, max_seqlen_k=max(lens),
+                                     cu_seqlens_k=cu, softmax_scale=d ** -0.5, causal=True)
+    at = 0
+    for n in lens:
+        qq = q[at:at + n].float().cpu().permute(1, 0, 2)
+        kk = k[at:at + n].float().cpu().permute(1, 0, 2).repeat_interleave(hq // hkv, 0)
+        vv = v[at:at + n].float().cpu().permute(1, 0, 2).repeat_interleave(hq // hkv, 0)
+        want = torch.nn.functional.scaled_dot_product_attention(qq, kk, vv, is_causal=True).permute(1, 0, 2)
+        assert (out[at:at + n].float().cpu() - want).abs().max() <= ATTN_ATOL
+        at += n
+    # strided K/V views of a fused qkv projection (infer/models/Qwen3.py:110-111) give the same result
+    qkv = torch.cat([q.reshape(t, -1), k.reshape(t, -1), v.reshape(t, -1)], dim=1)
+    _, k2, v2 = qkv.split([hq * d, hkv * d, hkv * d], dim=-1)
+    out2 = ops.flash_attn_varlen_func(q, k2.view(t, hkv, d), v2.view(t, hkv, d), max_seqlen_q=max(lens),
+                                      cu_seqlens_q=cu, max_seqlen_k=max(lens), cu_seqlens_k=cu, causal=True)
+    assert torch.equal(out, out2)
+
+
+def test_one_query_per_sequence_equals_decode(gpu):
+    wl = workloads.make_decode_workload("d", [37, 256, 700, 1023], 16, 8, nblk=16, seed=2).to(gpu)
+    dec = ops.flash_attn_with_kvcache(wl.q.unsqueeze(1), wl.k_cache, wl.v_cache, cache_seqlens=wl.context_lens,
+                                      block_table=wl.block_table, softmax_scale=wl.scale)[:, 0]
+    cu_q = torch.arange(5, dtype=torch.int32, device=gpu)
+    cu_k = torch.tensor(np.cumsum([0] + wl.lengths), dtype=torch.int32, device=gpu)
+    pre = ops.flash_attn_varlen_func(wl.q, wl.k_cache, wl.v_cache, max_seqlen_q=1, cu_seqlens_q=cu_q,
+                                     max_seqlen_k=1023, cu_seqlens_k=cu_k, softmax_scale=wl.scale, causal=True,
+                                     block_table=wl.block_table)
+    assert (pre.float() - dec.float()).abs().max() <= 4e-3     # two bf16 roundings of the same fp32 value
+
+
+def test_stale_nan_beyond_length_is_ignored(gpu):
+    wl = workloads.make_prefill_workload("p", [37, 300], [0, 256], 16, 8, seed=3, pad_fraction=0.0).to(gpu)
+    for i, n in enumerate(wl.lengths):
+        blk = int(wl.block_table[i, (n - 1) // 256])
+        wl.k_cache[blk, n % 256:] = float("nan")
+        wl.v_cache[blk, n % 256:] = float("nan")
+    out, kc, vc = run_paged(wl)
+    assert np.isfinite(f32(out)).all()
+    assert np.abs(f32(out) - oracle_paged(wl, kc, vc)).max() <= ATTN_ATOL
+
+
+def test_attention_module_prefill_then_decode(gpu):
+    """The reference's module-level flow (infer/ops/attention.py:96-122) on one layer: a prefill step
+    with a cached prefix, then a decode step for the same sequences."""
+    wl = workloads.make_prefill_workload("m", [300, 70], [256, 0], 16, 8, seed=9, pad_fraction=0.0).to(gpu)
+    att = Attention(16, 128, wl.scale, 8)
+    att.k_cache, att.v_cache = wl.k_cache.clone(), wl.v_cache.clone()
+    set_context(True, wl.cu_seqlens_q, wl.cu_seqlens_k, wl.max_seqlen_q, wl.max_seqlen_k, wl.slot_mapping, None,
+                wl.block_table)
+    o = att(wl.q.reshape(-1, 16 * 128), wl.k_new.reshape(-1, 8 * 128), wl.v_new.reshape(-1, 8 * 128))
+    want = oracle_paged(wl, att.k_cache, att.v_cache)
+    assert np.abs(f32(o).reshape(want.shape) - want).max() <= ATTN_ATOL
+    # decode one more token per sequence
+    g = torch.Generator().manual_seed(1)
+    q1 = torch.randn((2, 16 * 128), generator=g).to(torch.bfloat16).to(gpu)
+    k1 = torch.randn((2, 8 * 128), generator=g).to(torch.bfloat16).to(gpu)
+    v1 = torch.randn((2, 8 * 128), generator=g).to(torch.bfloat16).to(gpu)
+    lens = [n + 1 for n in wl.lengths]
+    slots = torch.tensor([int(wl.block_table[i, (n - 1) // 256]) * 256 + (n - 1) % 256 for i, n in enumerate(lens)],
+                         dtype=torch.int32, device=gpu)
+    ctx = torch.tensor(lens, dtype=torch.int32, device=gpu)
+    set_context(False, slot_mapping=slots, context_lens=ctx, block_tables=wl.block_table)
+    o1 = att(q1, k1, v1)
+    want1 = paged_ref.paged_decode_ref(bits(q1.view(2, 16, 128)), bits(att.k_cache), bits(att.v_cache),
+                                       wl.block_table.cpu().numpy(), ctx.cpu().numpy(), wl.scale)
+    assert np.abs(f32(o1).reshape(want1.shape) - want1).max() <= ATTN_ATOL
+    reset_context()
