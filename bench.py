@@ -164,6 +164,15 @@ def main():
     ap_ms = gpu_time_ms(append_step, max(args.steps, 48), reps)
     append_gbs = p3.append_bytes / (ap_ms * 1e-3) / 1e9
 
+    # paged varlen causal prefill attention on the same cfg3 step (after its append), for the record
+    kc3, vc3 = p3.k_cache.clone(), p3.v_cache.clone()
+    ops.store_kvcache(p3.k_new, p3.v_new, kc3, vc3, p3.slot_mapping)
+    pf_ms = gpu_time_ms(lambda: ops.flash_attn_varlen_func(
+        p3.q, kc3, vc3, max_seqlen_q=p3.max_seqlen_q, cu_seqlens_q=p3.cu_seqlens_q, max_seqlen_k=p3.max_seqlen_k,
+        cu_seqlens_k=p3.cu_seqlens_k, softmax_scale=p3.scale, causal=True, block_table=p3.block_table), 10, 2)
+    pairs = sum((n - c) * c + (n - c) * (n - c + 1) // 2 for n, c in zip(p3.lengths, p3.cached))
+    pf_flops = 4 * p3.num_q_heads * p3.head_dim * pairs
+
     line = {
         "metric": "paged decode attn HBM GB/s (% of 8 TB/s peak), Qwen3-8B shapes bs=64",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -183,6 +192,9 @@ def main():
                    "prefill_us": round(ap_ms * 1e3, 2), "prefill_GBps": round(append_gbs, 1),
                    "prefill_frac_of_peak": round(append_gbs / HBM_PEAK_GBS, 4)},
     }
+    line["prefill_attention"] = {"workload": "cfg3: 16 prompts U[64,2048], 0-50 % cached, causal over the paged cache",
+                                 "query_tokens": int(p3.q.shape[0]), "ms": round(pf_ms, 4),
+                                 "TFLOPs": round(pf_flops / (pf_ms * 1e-3) / 1e12, 1)}
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline()
     print(json.dumps(line))
