@@ -505,7 +505,7 @@ struct MergeArgs {
     int64_t out_stride0;
     const int32_t* ctx;
     int group;
-    const int32_t* header;
+    int split_workgroups;   // gridDim.x of the split launch that filled the workspace
     const int32_t* seg_first;
     const int32_t* seg_last;
     const float* ml;
@@ -513,48 +513,67 @@ struct MergeArgs {
     int batch;
 };
 
-// grid (batch, Hkv), 256 threads: each thread folds the segments of one (query head, 4 output
-// columns) item of its (sequence, KV head) with the running (max, sum) rule, loads of four
-// segments in flight at a time.
+// grid (batch, Hq), 256 threads = 8 segment lanes x 32 column quads.  Thread (j, c) folds segments
+// j, j + 8, ... of its (sequence, query head) for output columns 4c .. 4c+3 with the running
+// (max, sum) rule; the eight lanes are then folded through LDS.  All loads of a thread are
+// independent, so a sequence cut into many segments costs about one memory round trip.
 __global__ void __launch_bounds__(256) paged_decode_merge_kernel(MergeArgs a) {
+    __shared__ float red[8][32][6];
     const int b = blockIdx.x;
-    const int h = blockIdx.y;
+    const int head = blockIdx.y;
     const int G = a.group;
-    const bool empty = a.ctx[b] <= 0;
-    const int W = a.header[0];
-    const int w0 = empty ? 0 : a.seg_first[b];
-    const int w1 = empty ? -1 : a.seg_last[b];
-    const int64_t slot0 = (int64_t)h * (W + a.batch) + b;
-    for (int item = threadIdx.x; item < G * 32; item += 256) {
-        const int n = item >> 5, c4 = item & 31;
-        float m = -INFINITY, den = 0.f;
-        f32x4 num = {0.f, 0.f, 0.f, 0.f};
-        for (int wb = w0; wb <= w1; wb += 4) {
-            float2 mlv[4];
-            f32x4 pov[4];
+    const int h = head / G, n = head - h * G;
+    const int j = threadIdx.x >> 5, c4 = threadIdx.x & 31;
+    uint16_t* op = a.out + (int64_t)b * a.out_stride0 + (int64_t)head * kD + 4 * c4;
+    if (a.ctx[b] <= 0) {
+        if (j == 0) *reinterpret_cast<u32x2*>(op) = u32x2{0u, 0u};
+        return;
+    }
+    const int w0 = a.seg_first[b], w1 = a.seg_last[b];
+    const int64_t slot0 = (int64_t)h * (a.split_workgroups + a.batch) + b;
+    float m = -INFINITY, den = 0.f;
+    f32x4 num = {0.f, 0.f, 0.f, 0.f};
+    for (int wb = w0 + j; wb <= w1; wb += 32) {
+        float2 mlv[4];
+        f32x4 pov[4];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int wu = wb + u <= w1 ? wb + u : w1;
-                const int64_t row = (slot0 + wu) * G + n;
-                mlv[u] = *reinterpret_cast<const float2*>(a.ml + row * 2);
-                pov[u] = *reinterpret_cast<const f32x4*>(a.po + row * kD + 4 * c4);
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                if (wb + u > w1) break;
-                const float m_new = fmaxf(m, mlv[u].x);
-                const float f_old = __builtin_amdgcn_exp2f(m - m_new);
-                const float f_new = __builtin_amdgcn_exp2f(mlv[u].x - m_new);
-                den = den * f_old + mlv[u].y * f_new;
-                num = num * f_old + pov[u] * f_new;
-                m = m_new;
-            }
+        for (int u = 0; u < 4; ++u) {
+            const int wu = wb + 8 * u <= w1 ? wb + 8 * u : wb;
+            const int64_t row = (slot0 + wu) * G + n;
+            mlv[u] = *reinterpret_cast<const float2*>(a.ml + row * 2);
+            pov[u] = *reinterpret_cast<const f32x4*>(a.po + row * kD + 4 * c4);
         }
-        const float inv = den > 0.f ? 1.f / den : 0.f;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (wb + 8 * u > w1) break;
+            const float m_new = fmaxf(m, mlv[u].x);
+            const float f_old = __builtin_amdgcn_exp2f(m - m_new);
+            const float f_new = __builtin_amdgcn_exp2f(mlv[u].x - m_new);
+            den = den * f_old + mlv[u].y * f_new;
+            num = num * f_old + pov[u] * f_new;
+            m = m_new;
+        }
+    }
+    red[j][c4][0] = m; red[j][c4][1] = den;
+    red[j][c4][2] = num[0]; red[j][c4][3] = num[1]; red[j][c4][4] = num[2]; red[j][c4][5] = num[3];
+    __syncthreads();
+    if (j == 0) {
+        float mx = m;
+#pragma unroll
+        for (int k = 1; k < 8; ++k) mx = fmaxf(mx, red[k][c4][0]);
+        float d_tot = 0.f;
+        f32x4 n_tot = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float mk = red[k][c4][0];
+            const float f = mk == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mk - mx);
+            d_tot += red[k][c4][1] * f;
+            n_tot += f32x4{red[k][c4][2], red[k][c4][3], red[k][c4][4], red[k][c4][5]} * f;
+        }
+        const float inv = d_tot > 0.f ? 1.f / d_tot : 0.f;
         union { __bf16 hv[4]; u32x2 u; } r;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) r.hv[e] = (__bf16)(num[e] * inv);
-        uint16_t* op = a.out + (int64_t)b * a.out_stride0 + (int64_t)(h * G + n) * kD + 4 * c4;
+        for (int e = 0; e < 4; ++e) r.hv[e] = (__bf16)(n_tot[e] * inv);
         *reinterpret_cast<u32x2*>(op) = r.u;
     }
 }
@@ -694,19 +713,22 @@ int infer_paged_decode_merge_bf16(void* out, int64_t out_stride0, const int32_t*
     const int G = (int)(num_q_heads / num_kv_heads);
     DecodeWorkspace ws = decode_workspace_layout(batch, G, num_kv_heads);
     if (ws.total_bytes > workspace_bytes) return INFER_KV_EWORKSPACE;
+    Launch L;
+    int rc = plan_launch(num_kv_heads, &L);   // same knob -> same split count as the split launch
+    if (rc) return rc;
     const char* base = (const char*)workspace;
     MergeArgs m;
     m.out = (uint16_t*)out;
     m.out_stride0 = out_stride0;
     m.ctx = context_lens;
     m.group = G;
-    m.header = (const int32_t*)(base + ws.header_off);
+    m.split_workgroups = L.W;
     m.seg_first = (const int32_t*)(base + ws.seg_first_off);
     m.seg_last = (const int32_t*)(base + ws.seg_last_off);
     m.ml = (const float*)(base + ws.ml_off);
     m.po = (const float*)(base + ws.po_off);
     m.batch = (int)batch;
-    dim3 grid((unsigned)batch, (unsigned)num_kv_heads, 1), block(256, 1, 1);
+    dim3 grid((unsigned)batch, (unsigned)num_q_heads, 1), block(256, 1, 1);
     hipLaunchKernelGGL(paged_decode_merge_kernel, grid, block, 0, (hipStream_t)stream, m);
     return (int)hipGetLastError();
 }
