@@ -139,6 +139,33 @@ def test_large_batch(gpu):
     check(wl)
 
 
+@pytest.mark.parametrize("splits", [4, 40, None])
+def test_many_tiny_sequences_in_one_span(gpu, splits):
+    """Hundreds of sequences shorter than a span: one wavefront walks many segments, more than fit its
+    LDS plan table (32) or its parked-partials area (4 at group size 4), so the batching and the
+    early-drain paths run."""
+    g = torch.Generator().manual_seed(21)
+    lens = torch.randint(1, 70, (900,), generator=g).tolist()
+    wl = workloads.make_decode_workload("tiny900", lens, 32, 8, bs=32, seed=21).to(gpu)
+    check(wl, splits=splits)
+
+
+@pytest.mark.parametrize("hq", [8, 64, 128])
+def test_many_short_sequences_other_group_sizes(gpu, hq):
+    g = torch.Generator().manual_seed(22)
+    lens = torch.randint(1, 100, (200,), generator=g).tolist()
+    wl = workloads.make_decode_workload("short200", lens, hq, 8, bs=32, seed=22).to(gpu)
+    check(wl, splits=8)
+
+
+def test_one_span_longer_than_64_blocks(gpu):
+    """A single wavefront streaming 150 blocks of one sequence: block ids past the 64 held in the
+    lane-indexed register come from the table directly."""
+    wl = workloads.make_decode_workload("long1", [4800, 33], 16, 8, bs=32, nblk=160, seed=23).to(gpu)
+    check(wl, splits=1)
+    check(wl, splits=2)
+
+
 def test_cfg2_full_size(gpu):
     wl = workloads.cfg2(device=gpu)
     err = check(wl)
