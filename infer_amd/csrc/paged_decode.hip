@@ -37,6 +37,9 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef short i16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
 
 constexpr int kD = 128;            // head_dim
 constexpr int kStep = 32;          // tokens per step
@@ -211,11 +214,12 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
     float m_run = -INFINITY;
     float l_run = 0.f;
 
-    // Row r of a K tile holds token 4 (r % 4) + r / 4 of the tile, so that result element
-    // (tile t, quad element e) of lane group g is token 4 (4 t + e) + g of the step.
-    const uint32_t k_lane = (uint32_t)((4 * (n & 3) + (n >> 2)) * a.tok_stride + 8 * g);
+    // Row r of K tile t holds token 8 (r / 4) + 4 t + r % 4 of the step, so that result element
+    // (tile t, quad element e) of lane group g is token 8 g + (4 t + e): lane group g ends up with
+    // the 8 consecutive tokens 8 g .. 8 g + 7, which is also how the transposing LDS read hands out V.
+    const uint32_t k_lane = (uint32_t)((8 * (n >> 2) + (n & 3)) * a.tok_stride + 8 * g);
     const uint32_t v_lane = (uint32_t)(g * a.tok_stride + 8 * n);
-    const uint32_t tile_off = (uint32_t)(16 * a.tok_stride);
+    const uint32_t tile_off = (uint32_t)(4 * a.tok_stride);
     const uint32_t quad_off = (uint32_t)(4 * a.tok_stride);
     const uint16_t* dummy = a.q;   // 256 readable bytes that stay in cache
 
@@ -325,7 +329,7 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
         if (tail) {
 #pragma unroll
             for (int i = 0; i < 8; ++i)
-                if (tok0 + 4 * i + g >= len) sv[i] = -INFINITY;
+                if (tok0 + 8 * g + i >= len) sv[i] = -INFINITY;
         }
         float mx = sv[0];
 #pragma unroll
@@ -364,18 +368,16 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
 #pragma unroll
             for (int t = 0; t < 8; ++t) acc[t] *= alpha;
         }
-        // ---- O^T += V^T P^T : A operand element i of lane (g, n) is V[token 4 i + g][16 t + n]
+        // ---- O^T += V^T P^T : A operand element i of lane (g, n) is V[token 8 g + i][16 t + n].
+        // ds_read_b64_tr_b16: in each group of 16 lanes, lane i points at 4 consecutive elements of
+        // row i / 4 (column quad i % 4) and lane l receives column l of those four rows.
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            const unsigned char* col = lds + g * kLdsRow + (16 * t + n) * 2;
-            u32x4 vt;
-#pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                uint32_t lo = *reinterpret_cast<const uint16_t*>(col + (8 * p) * kLdsRow);
-                uint32_t hi = *reinterpret_cast<const uint16_t*>(col + (8 * p + 4) * kLdsRow);
-                vt[p] = lo | (hi << 16);
-            }
-            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vt), pb, acc[t], 0, 0, 0);
+            const unsigned char* src = lds + (8 * g + (n >> 2)) * kLdsRow + (16 * t + 4 * (n & 3)) * 2;
+            const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src));
+            const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src + 4 * kLdsRow));
+            const i16x8 vt = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vt), pb, acc[t], 0, 0, 0);
         }
         lds_order();
 
