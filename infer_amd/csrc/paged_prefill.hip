@@ -25,6 +25,9 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef short i16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
 
 constexpr int kD = 128;
 constexpr int kStep = 32;        // keys per step
@@ -101,7 +104,8 @@ __global__ void __launch_bounds__(1024) paged_prefill_kernel(PrefillArgs a) {
     for (int t = 0; t < 8; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
 
-    const int krow = 4 * (n & 3) + (n >> 2);   // row r of a K tile holds key 4 (r % 4) + r / 4 of the tile
+    // row r of K tile t holds key 8 (r / 4) + 4 t + r % 4 of the step: lane group g ends up with keys 8 g .. 8 g + 7
+    const int krow = 8 * (n >> 2) + (n & 3);
     u32x4 kreg[2][4];
     u32x4 vreg[8];
 
@@ -115,7 +119,7 @@ __global__ void __launch_bounds__(1024) paged_prefill_kernel(PrefillArgs a) {
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                    kreg[t][j] = load16(a.k + base + (int64_t)(16 * t + krow) * a.tok_stride + 8 * g + 32 * j);
+                    kreg[t][j] = load16(a.k + base + (int64_t)(4 * t + krow) * a.tok_stride + 8 * g + 32 * j);
 #pragma unroll
             for (int i = 0; i < 8; ++i) vreg[i] = load16(a.v + base + (int64_t)(4 * i + g) * a.tok_stride + 8 * n);
         } else {
@@ -123,7 +127,7 @@ __global__ void __launch_bounds__(1024) paged_prefill_kernel(PrefillArgs a) {
             const int64_t last = a.total_k_rows - 1;
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-                int64_t r = row0 + 16 * t + krow;
+                int64_t r = row0 + 4 * t + krow;
                 r = r > last ? last : r;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) kreg[t][j] = load16(a.k + r * a.tok_stride + (int64_t)kvh * kD + 8 * g + 32 * j);
@@ -168,7 +172,7 @@ __global__ void __launch_bounds__(1024) paged_prefill_kernel(PrefillArgs a) {
         if (tok0 + kStep - 1 > my_limit) {
 #pragma unroll
             for (int i = 0; i < 8; ++i)
-                if (tok0 + 4 * i + g > my_limit) sv[i] = -INFINITY;
+                if (tok0 + 8 * g + i > my_limit) sv[i] = -INFINITY;
         }
         float mx = sv[0];
 #pragma unroll
@@ -195,17 +199,16 @@ __global__ void __launch_bounds__(1024) paged_prefill_kernel(PrefillArgs a) {
 #pragma unroll
             for (int t = 0; t < 8; ++t) acc[t] *= alpha;
         }
+        // A operand element i of lane (g, n) is V[key 8 g + i][16 t + n], fetched with the transposing
+        // LDS read: in each group of 16 lanes, lane i points at row i / 4, column quad i % 4, and lane l
+        // receives column l of those four rows.
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            const unsigned char* col = lds + g * kLdsRow + (16 * t + n) * 2;
-            u32x4 vt;
-#pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                uint32_t lo = *reinterpret_cast<const uint16_t*>(col + (8 * p) * kLdsRow);
-                uint32_t hi = *reinterpret_cast<const uint16_t*>(col + (8 * p + 4) * kLdsRow);
-                vt[p] = lo | (hi << 16);
-            }
-            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vt), pb, acc[t], 0, 0, 0);
+            const unsigned char* src = lds + (8 * g + (n >> 2)) * kLdsRow + (16 * t + 4 * (n & 3)) * 2;
+            const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src));
+            const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src + 4 * kLdsRow));
+            const i16x8 vt = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vt), pb, acc[t], 0, 0, 0);
         }
         lds_order();
     }
