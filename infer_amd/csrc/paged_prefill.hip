@@ -228,6 +228,219 @@ __global__ void __launch_bounds__(1024) paged_prefill_kernel(PrefillArgs a) {
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Tiled variant, used when the GQA group size is 1, 2, 4 or 8: the WAVES = G wavefronts of a
+// workgroup (one query head each, 32 queries = 2 MFMA column tiles) share every 32-key K tile and
+// V tile through LDS.  The tiles are fetched once per workgroup with fully coalesced 16-byte loads,
+// double-buffered (global loads of tile s+1 are in flight while tile s is consumed; one barrier per
+// step), so cache traffic per query drops by 2 G against the one-wave-per-tile kernel above.
+constexpr int kNQ = 2;
+constexpr int kQBlock = kNQ * kQTile;
+constexpr int kTileBytes = kStep * kLdsRow;
+
+template <int WAVES>
+__global__ void __launch_bounds__(64 * WAVES) paged_prefill_tile_kernel(PrefillArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_all[];   // [2][K tile | V tile]
+    constexpr int kThreads = 64 * WAVES;
+    constexpr int kChunks = 512 / kThreads;        // 16-byte chunks of a 32 x 256 B tile per thread
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 4, n = lane & 15;
+    const int b = blockIdx.y;
+    const int kvh = blockIdx.z;
+    const int head = kvh * WAVES + wave;
+
+    const int q_beg = a.cu_q[b], q_end = a.cu_q[b + 1];
+    const int k_beg = a.cu_k[b], k_end = a.cu_k[b + 1];
+    const int sq = q_end - q_beg, sk = k_end - k_beg;
+    const int q0 = blockIdx.x * kQBlock;
+    if (q0 >= sq) return;
+    if (sk <= 0) {
+#pragma unroll
+        for (int u = 0; u < kNQ; ++u)
+            if (q0 + 16 * u + n < sq) {
+                uint16_t* op = a.out + (int64_t)(q_beg + q0 + 16 * u + n) * a.out_stride0 + (int64_t)head * kD + 4 * g;
+                for (int t = 0; t < 8; ++t) *reinterpret_cast<u32x2*>(op + 16 * t) = u32x2{0u, 0u};
+            }
+        return;
+    }
+    const int shift = sk - sq;
+    int my_q[kNQ], my_limit[kNQ];
+#pragma unroll
+    for (int u = 0; u < kNQ; ++u) {
+        my_q[u] = q0 + 16 * u + n;
+        my_limit[u] = a.causal ? (my_q[u] + shift < sk - 1 ? my_q[u] + shift : sk - 1) : sk - 1;
+    }
+    const int block_last = q0 + kQBlock - 1 < sq - 1 ? q0 + kQBlock - 1 : sq - 1;
+    const int key_end = a.causal ? (block_last + shift + 1 < sk ? block_last + shift + 1 : sk) : sk;
+    const int nsteps = (key_end + kStep - 1) / kStep;
+
+    bf16x8 qreg[kNQ][4];
+#pragma unroll
+    for (int u = 0; u < kNQ; ++u) {
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        const bool live = my_q[u] < sq;
+        const uint16_t* qp = a.q + (int64_t)(q_beg + (live ? my_q[u] : 0)) * a.q_stride0 + (int64_t)head * kD + 8 * g;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) qreg[u][j] = as_bf16x8(live ? load16(qp + 32 * j) : z);
+    }
+    f32x4 acc[kNQ][8];
+    float m_run[kNQ], l_run[kNQ];
+#pragma unroll
+    for (int u = 0; u < kNQ; ++u) {
+#pragma unroll
+        for (int t = 0; t < 8; ++t) acc[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        m_run[u] = -INFINITY;
+        l_run[u] = 0.f;
+    }
+
+    // cooperative tile fetch: chunk c covers bytes [16 (c % 16), +16) of row c / 16
+    u32x4 kst[kChunks], vst[kChunks];
+    auto fetch = [&](int s) {
+        const int tok0 = s * kStep;
+        int64_t base = 0;
+        if (a.bt) {
+            int blk = __builtin_amdgcn_readfirstlane(a.bt[(int64_t)b * a.bt_stride0 + tok0 / a.block_size]);
+            blk = blk < 0 ? 0 : (blk >= a.num_blocks ? a.num_blocks - 1 : blk);
+            base = (int64_t)blk * a.blk_stride + (int64_t)(tok0 % a.block_size) * a.tok_stride;
+        }
+#pragma unroll
+        for (int i = 0; i < kChunks; ++i) {
+            const int c = tid + i * kThreads;
+            const int r = c >> 4, col = (c & 15) * 8;
+            int64_t off;
+            if (a.bt) off = base + (int64_t)r * a.tok_stride;
+            else {
+                int64_t row = (int64_t)k_beg + tok0 + r;
+                row = row > a.total_k_rows - 1 ? a.total_k_rows - 1 : row;
+                off = row * a.tok_stride;
+            }
+            off += (int64_t)kvh * kD + col;
+            const bool valid = tok0 + r < sk;      // rows past the sequence may hold anything: read as zeros
+            const u32x4 z = {0u, 0u, 0u, 0u};
+            kst[i] = valid ? load16(a.k + off) : z;
+            vst[i] = valid ? load16(a.v + off) : z;
+        }
+    };
+    auto stash = [&](int buf) {
+        unsigned char* kb = lds_all + buf * 2 * kTileBytes;
+#pragma unroll
+        for (int i = 0; i < kChunks; ++i) {
+            const int c = tid + i * kThreads;
+            const int off = (c >> 4) * kLdsRow + (c & 15) * 16;
+            *reinterpret_cast<u32x4*>(kb + off) = kst[i];
+            *reinterpret_cast<u32x4*>(kb + kTileBytes + off) = vst[i];
+        }
+    };
+
+    fetch(0);
+    stash(0);
+    __syncthreads();
+
+    // K operand row of this lane inside a tile: row r of K tile t holds key 8 (r / 4) + 4 t + r % 4
+    const int krow = 8 * (n >> 2) + (n & 3);
+    for (int s = 0; s < nsteps; ++s) {
+        if (s + 1 < nsteps) fetch(s + 1);
+        const unsigned char* kb = lds_all + (s & 1) * 2 * kTileBytes;
+        const unsigned char* vb = kb + kTileBytes;
+        const int tok0 = s * kStep;
+
+        // ---- S^T = K Q^T for both query tiles
+        f32x4 sc[kNQ][2];
+#pragma unroll
+        for (int u = 0; u < kNQ; ++u)
+#pragma unroll
+            for (int t = 0; t < 2; ++t) sc[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const u32x4 kf = *reinterpret_cast<const u32x4*>(kb + (4 * t + krow) * kLdsRow + (32 * j + 8 * g) * 2);
+#pragma unroll
+                for (int u = 0; u < kNQ; ++u)
+                    sc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf), qreg[u][j], sc[u][t], 0, 0, 0);
+            }
+
+        // ---- online softmax per query tile
+        bf16x8 pb[kNQ];
+#pragma unroll
+        for (int u = 0; u < kNQ; ++u) {
+            float sv[8];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sv[4 * t + e] = sc[u][t][e] * a.scale_log2;
+            if (tok0 + kStep - 1 > my_limit[u]) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    if (tok0 + 8 * g + i > my_limit[u]) sv[i] = -INFINITY;
+            }
+            float mx = sv[0];
+#pragma unroll
+            for (int i = 1; i < 8; ++i) mx = fmaxf(mx, sv[i]);
+            mx = fmaxf(mx, __shfl_xor(mx, 16));
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float m_new = fmaxf(m_run[u], mx);
+            const float m_ref = m_new == -INFINITY ? 0.f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m_run[u] - m_ref);
+            m_run[u] = m_new;
+            float psum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float p = __builtin_amdgcn_exp2f(sv[i] - m_ref);
+                psum += p;
+                pb[u][i] = (__bf16)p;
+            }
+            l_run[u] = l_run[u] * alpha + psum;
+            if (__any(alpha != 1.f)) {
+#pragma unroll
+                for (int t = 0; t < 8; ++t) acc[u][t] *= alpha;
+            }
+        }
+
+        // ---- O^T += V^T P^T, every V fragment used for both query tiles
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const unsigned char* src = vb + (8 * g + (n >> 2)) * kLdsRow + (16 * t + 4 * (n & 3)) * 2;
+            const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src));
+            const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src + 4 * kLdsRow));
+            const bf16x8 vt = __builtin_bit_cast(bf16x8, (i16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+#pragma unroll
+            for (int u = 0; u < kNQ; ++u)
+                acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pb[u], acc[u][t], 0, 0, 0);
+        }
+
+        if (s + 1 < nsteps) stash((s + 1) & 1);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int u = 0; u < kNQ; ++u) {
+        float l = l_run[u] + __shfl_xor(l_run[u], 16);
+        l += __shfl_xor(l, 32);
+        if (my_q[u] < sq) {
+            const float inv = l > 0.f ? 1.f / l : 0.f;
+            uint16_t* op = a.out + (int64_t)(q_beg + my_q[u]) * a.out_stride0 + (int64_t)head * kD + 4 * g;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                union { __bf16 hv[4]; u32x2 w; } r;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) r.hv[e] = (__bf16)(acc[u][t][e] * inv);
+                *reinterpret_cast<u32x2*>(op + 16 * t) = r.w;
+            }
+        }
+    }
+}
+
+template <int WAVES>
+int launch_tiled(const PrefillArgs& a, int64_t max_seqlen_q, int64_t num_seqs, int64_t num_kv_heads, hipStream_t st) {
+    dim3 grid((unsigned)((max_seqlen_q + kQBlock - 1) / kQBlock), (unsigned)num_seqs, (unsigned)num_kv_heads);
+    hipLaunchKernelGGL(paged_prefill_tile_kernel<WAVES>, grid, dim3(64 * WAVES, 1, 1), 4 * kTileBytes, st, a);
+    return (int)hipGetLastError();
+}
+
 }  // namespace
 
 extern "C" int infer_paged_prefill_bf16(const void* q, int64_t q_stride0, const void* k, const void* v,
@@ -260,6 +473,13 @@ extern "C" int infer_paged_prefill_bf16(const void* q, int64_t q_stride0, const 
     a.total_k_rows = kv_rows;
     a.scale_log2 = scale * 1.4426950408889634f;
     a.causal = causal ? 1 : 0;
+    switch (G) {   // group sizes with a shared-tile kernel
+        case 1: return launch_tiled<1>(a, max_seqlen_q, num_seqs, num_kv_heads, (hipStream_t)stream);
+        case 2: return launch_tiled<2>(a, max_seqlen_q, num_seqs, num_kv_heads, (hipStream_t)stream);
+        case 4: return launch_tiled<4>(a, max_seqlen_q, num_seqs, num_kv_heads, (hipStream_t)stream);
+        case 8: return launch_tiled<8>(a, max_seqlen_q, num_seqs, num_kv_heads, (hipStream_t)stream);
+        default: break;
+    }
     const size_t lds_bytes = (size_t)G * kLdsWave;
     static bool attr_set = false;
     if (!attr_set) {
