@@ -255,7 +255,8 @@ __global__ void __launch_bounds__(64 * WAVES) paged_prefill_tile_kernel(PrefillA
     const int q_beg = a.cu_q[b], q_end = a.cu_q[b + 1];
     const int k_beg = a.cu_k[b], k_end = a.cu_k[b + 1];
     const int sq = q_end - q_beg, sk = k_end - k_beg;
-    const int q0 = blockIdx.x * kQBlock;
+    // late query blocks see the most keys: hand them out first so the long workgroups start early
+    const int q0 = (int)(gridDim.x - 1 - blockIdx.x) * kQBlock;
     if (q0 >= sq) return;
     if (sk <= 0) {
 #pragma unroll
