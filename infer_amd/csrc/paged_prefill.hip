@@ -17,6 +17,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "../../include/infer_kv.h"
 
 namespace {
@@ -298,8 +300,10 @@ __global__ void __launch_bounds__(64 * WAVES) paged_prefill_tile_kernel(PrefillA
     }
 
     // cooperative tile fetch: chunk c covers bytes [16 (c % 16), +16) of row c / 16
-    u32x4 kst[kChunks], vst[kChunks];
-    auto fetch = [&](int s) {
+    // two tiles are in flight in registers (slots 0 and 1 alternate), a third is being consumed from LDS
+    u32x4 kst[2][kChunks], vst[2][kChunks];
+    auto fetch = [&](auto SLOT, int s) {
+        constexpr int S = decltype(SLOT)::value;
         const int tok0 = s * kStep;
         int64_t base = 0;
         if (a.bt) {
@@ -321,29 +325,36 @@ __global__ void __launch_bounds__(64 * WAVES) paged_prefill_tile_kernel(PrefillA
             off += (int64_t)kvh * kD + col;
             const bool valid = tok0 + r < sk;      // rows past the sequence may hold anything: read as zeros
             const u32x4 z = {0u, 0u, 0u, 0u};
-            kst[i] = valid ? load16(a.k + off) : z;
-            vst[i] = valid ? load16(a.v + off) : z;
+            kst[S][i] = valid ? load16(a.k + off) : z;
+            vst[S][i] = valid ? load16(a.v + off) : z;
         }
     };
-    auto stash = [&](int buf) {
+    auto stash = [&](auto SLOT, int buf) {
+        constexpr int S = decltype(SLOT)::value;
         unsigned char* kb = lds_all + buf * 2 * kTileBytes;
 #pragma unroll
         for (int i = 0; i < kChunks; ++i) {
             const int c = tid + i * kThreads;
             const int off = (c >> 4) * kLdsRow + (c & 15) * 16;
-            *reinterpret_cast<u32x4*>(kb + off) = kst[i];
-            *reinterpret_cast<u32x4*>(kb + kTileBytes + off) = vst[i];
+            *reinterpret_cast<u32x4*>(kb + off) = kst[S][i];
+            *reinterpret_cast<u32x4*>(kb + kTileBytes + off) = vst[S][i];
         }
     };
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
 
-    fetch(0);
-    stash(0);
+    // tile s travels in slot s % 2: fetched during step s - 2, stored to LDS at the end of step s - 1
+    fetch(S0{}, 0);
+    if (nsteps > 1) fetch(S1{}, 1);
+    stash(S0{}, 0);
     __syncthreads();
 
     // K operand row of this lane inside a tile: row r of K tile t holds key 8 (r / 4) + 4 t + r % 4
     const int krow = 8 * (n >> 2) + (n & 3);
-    for (int s = 0; s < nsteps; ++s) {
-        if (s + 1 < nsteps) fetch(s + 1);
+    auto step = [&](auto SLOT, int s) {
+        constexpr int S = decltype(SLOT)::value;          // slot of tile s (just consumed from LDS): free again
+        using NEXT = std::integral_constant<int, 1 - S>;  // slot of tile s + 1
+        if (s + 2 < nsteps) fetch(SLOT, s + 2);
         const unsigned char* kb = lds_all + (s & 1) * 2 * kTileBytes;
         const unsigned char* vb = kb + kTileBytes;
         const int tok0 = s * kStep;
@@ -413,8 +424,16 @@ __global__ void __launch_bounds__(64 * WAVES) paged_prefill_tile_kernel(PrefillA
                 acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pb[u], acc[u][t], 0, 0, 0);
         }
 
-        if (s + 1 < nsteps) stash((s + 1) & 1);
+        if (s + 1 < nsteps) stash(NEXT{}, (s + 1) & 1);
         __syncthreads();
+    };
+    {
+        int s = 0;
+        for (; s + 1 < nsteps; s += 2) {
+            step(S0{}, s);
+            step(S1{}, s + 1);
+        }
+        if (s < nsteps) step(S0{}, s);
     }
 
 #pragma unroll
