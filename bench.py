@@ -78,6 +78,9 @@ def main():
     ap.add_argument("--copies", type=int, default=4, help="independent cache copies walked round-robin")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--splits", type=int, default=0, help="KV-split workgroups (0 = library default)")
+    ap.add_argument("--ceiling", action="store_true",
+                    help="measure what this GPU sustains for a read-only stream and a copy (plain kernels of the "
+                         "library, same timing method) and print it as JSON; no KV-cache kernel runs")
     ap.add_argument("--counters", action="store_true",
                     help="short untimed run for `rocprofv3 --pmc`: a 1 GiB plain copy (x3), the decode op (x5), "
                          "a prefill-sized append (x3)")
@@ -92,6 +95,39 @@ def main():
 
     from infer_amd import ops, workloads
     dev = torch.device("cuda:0")
+    if args.ceiling:
+        from infer_amd import _lib
+        lib = _lib.load()
+        stream = torch.cuda.current_stream().cuda_stream
+        sink = torch.zeros(4, dtype=torch.uint8, device=dev)
+        res = {"ceiling_run": True, "method": "HIP events, 30 launches after 3 warm-ups, buffers rotated (4 x size)"}
+        for label, nbytes in (("640MB", 640 * 10 ** 6 // 16 * 16), ("2GiB", 1 << 31)):
+            bufs = [torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(4)]
+            dst = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            it = [0]
+
+            def rd(wg):
+                def f():
+                    i = it[0] % 4
+                    it[0] += 1
+                    _lib.check(lib.infer_kv_probe_read(bufs[i].data_ptr(), nbytes, sink.data_ptr(), wg, stream), "probe")
+                return f
+
+            def cp(wg):
+                def f():
+                    i = it[0] % 4
+                    it[0] += 1
+                    _lib.check(lib.infer_kv_probe_copy(bufs[i].data_ptr(), dst.data_ptr(), nbytes, wg, stream), "probe")
+                return f
+            for wg in (256, 512, 1024):
+                ms = gpu_time_ms(rd(wg), 30, 3)
+                res[f"read_{label}_{wg}wg_GBps"] = round(nbytes / ms / 1e6, 1)
+            for wg in (2048, 8192):
+                ms = gpu_time_ms(cp(wg), 30, 3)
+                res[f"copy_{label}_{wg}wg_GBps_read_plus_write"] = round(2 * nbytes / ms / 1e6, 1)
+            del bufs, dst
+        print(json.dumps(res))
+        return
     if args.splits:
         ops.set_split_workgroups(args.splits)
     wl = workloads.cfg2(device=dev)

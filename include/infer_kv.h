@@ -159,6 +159,13 @@ int infer_paged_prefill_bf16(const void* q, int64_t q_stride0,
  * (0 = choose from the device's CU count).  Process-wide; returns the previous value. */
 int infer_paged_decode_set_split_workgroups(int workgroups);
 
+/* ------------------------------------------------------------------ measurement helpers
+ * No counterpart in the reference.  Plain streaming kernels used by bench.py --ceiling to measure
+ * what the part sustains for a read-only stream (same launch shape as the decode kernel: one
+ * 512-thread workgroup per contiguous share) and for a copy.  `sink4` is 4 writable bytes. */
+int infer_kv_probe_read(const void* src, size_t bytes, void* sink4, int workgroups, void* stream);
+int infer_kv_probe_copy(const void* src, void* dst, size_t bytes, int workgroups, void* stream);
+
 /* ------------------------------------------------------------------ 3. block pool (host only)
  * C view of infer::BlockPool (include/infer_kv/block_pool.hpp), the native counterpart of the
  * reference's Python BlockManager (infer/engine/block_mannager.py:44-133), which is the block

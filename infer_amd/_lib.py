@@ -33,6 +33,8 @@ SIGNATURES = {
     "infer_paged_decode_set_split_workgroups": (_c.c_int, [_c.c_int]),
     "infer_paged_prefill_bf16": (_c.c_int, [_vp, _i64, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _i64,
                                             _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _c.c_int, _vp]),
+    "infer_kv_probe_read": (_c.c_int, [_vp, _sz, _vp, _c.c_int, _vp]),
+    "infer_kv_probe_copy": (_c.c_int, [_vp, _vp, _sz, _c.c_int, _vp]),
     "infer_pool_create": (_vp, [_i32, _i32]),
     "infer_pool_destroy": (None, [_vp]),
     "infer_pool_last_error": (_c.c_char_p, []),

@@ -1,0 +1,64 @@
+// Streaming probes: what this GPU sustains for a read-only stream and for a plain copy, measured
+// with the same launch shape as the decode kernel (one workgroup of 512 threads per span, 16-byte
+// loads, three batches of eight loads in flight per lane).  Not part of the KV-cache path; bench.py
+// --ceiling uses it to put the kernels' achieved bandwidth next to the practical ceiling of the part.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/infer_kv.h"
+
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t fold(u32x4 a) { return a.x ^ a.y ^ a.z ^ a.w; }
+
+// Each workgroup reads a contiguous share of the buffer exactly once.
+__global__ void __launch_bounds__(512) stream_read_kernel(const u32x4* __restrict__ src, size_t n_vec, uint32_t* sink) {
+    const size_t per = n_vec / gridDim.x;
+    const u32x4* p = src + per * blockIdx.x;
+    uint32_t acc = 0;
+    size_t i = threadIdx.x;
+    for (; i + 7 * 512 < per; i += 8 * 512) {
+        u32x4 r[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) r[u] = p[i + u * 512];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc ^= fold(r[u]);
+    }
+    for (; i < per; i += 512) acc ^= fold(p[i]);
+    if (acc == 0x9e3779b9u) *sink = acc;   // keeps the loads alive; practically never true
+}
+
+__global__ void __launch_bounds__(256) stream_copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, size_t n_vec) {
+    const size_t stride = (size_t)gridDim.x * 256;
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    for (; i + 3 * stride < n_vec; i += 4 * stride) {
+        u32x4 r[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) r[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) __builtin_nontemporal_store(r[u], dst + i + u * stride);
+    }
+    for (; i < n_vec; i += stride) dst[i] = src[i];
+}
+
+}  // namespace
+
+extern "C" {
+
+int infer_kv_probe_read(const void* src, size_t bytes, void* sink4, int workgroups, void* stream) {
+    if (!src || !sink4 || bytes < 16 || workgroups <= 0 || ((uintptr_t)src & 15)) return INFER_KV_EINVAL;
+    hipLaunchKernelGGL(stream_read_kernel, dim3(workgroups), dim3(512), 0, (hipStream_t)stream, (const u32x4*)src,
+                       bytes / 16, (uint32_t*)sink4);
+    return (int)hipGetLastError();
+}
+
+int infer_kv_probe_copy(const void* src, void* dst, size_t bytes, int workgroups, void* stream) {
+    if (!src || !dst || bytes < 16 || workgroups <= 0 || (((uintptr_t)src | (uintptr_t)dst) & 15)) return INFER_KV_EINVAL;
+    hipLaunchKernelGGL(stream_copy_kernel, dim3(workgroups), dim3(256), 0, (hipStream_t)stream, (const u32x4*)src,
+                       (u32x4*)dst, bytes / 16);
+    return (int)hipGetLastError();
+}
+
+}  // extern "C"
