@@ -57,6 +57,11 @@ public:
     // the last block when the new token filled it.
     void may_append(const int64_t* token_ids, int64_t seq_len, std::vector<int32_t>& table);
 
+    // Raw allocation without token ids (no prefix sharing), for callers that only know lengths:
+    // takes the block at the front of the free FIFO / drops one reference.
+    int32_t acquire_block();
+    void release_block(int32_t block_id);
+
     // introspection for tests and statistics
     int32_t ref_count(int32_t block_id) const;
     bool has_hash(int32_t block_id) const;

@@ -235,6 +235,20 @@ void BlockPool::may_append(const int64_t* token_ids, int64_t seq_len, std::vecto
     }
 }
 
+int32_t BlockPool::acquire_block() {
+    std::lock_guard<std::mutex> g(mu_);
+    if (free_head_ < 0) throw std::logic_error("BlockPool::acquire_block: out of blocks");
+    const int32_t id = free_head_;
+    take(id);
+    return id;
+}
+
+void BlockPool::release_block(int32_t id) {
+    std::lock_guard<std::mutex> g(mu_);
+    if (id < 0 || id >= num_blocks_ || blocks_[id].ref_count <= 0) throw std::logic_error("BlockPool::release_block: block not held");
+    if (--blocks_[id].ref_count == 0) release(id);
+}
+
 int32_t BlockPool::ref_count(int32_t id) const { std::lock_guard<std::mutex> g(mu_); return blocks_.at(id).ref_count; }
 bool BlockPool::has_hash(int32_t id) const { std::lock_guard<std::mutex> g(mu_); return blocks_.at(id).hashed; }
 uint64_t BlockPool::block_hash(int32_t id) const { std::lock_guard<std::mutex> g(mu_); return blocks_.at(id).hash; }
