@@ -65,6 +65,30 @@ int infer_kv_append_bf16(const void* key, int64_t key_stride0,
                          int64_t n_rows, int64_t dkv, int64_t num_slots,
                          void* stream);
 
+/* ------------------------------------------------------------------ 1b. fused QK-norm + RoPE + KV append
+ * Replaces, in one launch, the four steps in front of attention in QwenAttention.forward
+ * (infer/models/Qwen3.py:113-131): q_norm and k_norm (RMSNorm.rms_forward, infer/ops/norm.py:63-73,
+ * per head over head_dim with a [head_dim] bf16 weight), the in-place neox rotary embedding
+ * (rotary_embedding_kernel, src/operators/rope/rope.cu:43-133; rot_dim == head_dim) and
+ * store_kvcache (infer/ops/attention.py:16-45).
+ *
+ * q [n_rows, Hq, D] and k [n_rows, Hkv, D] (row strides in elements, heads contiguous) are
+ * normalised and rotated; q is updated in place; the new k row goes to k_cache[slot] and, when
+ * write_k_inplace != 0, also back into k; the v row is copied to v_cache[slot].  Rows whose slot is
+ * negative or >= num_slots update q (and k in place) only.  positions are int64 and are clamped
+ * into [0, max_position); cos_sin_cache is [max_position, D] bf16 = cos(D/2) | sin(D/2) per row.
+ * Arithmetic rounds where the reference rounds (see the kernel source).  head_dim must be 128.
+ */
+int infer_kv_qk_norm_rope_append_bf16(void* q, int64_t q_stride0, void* k, int64_t k_stride0,
+                                      const void* v, int64_t v_stride0,
+                                      const int64_t* positions,
+                                      const void* q_norm_weight, const void* k_norm_weight, float eps,
+                                      const void* cos_sin_cache, int64_t max_position,
+                                      void* k_cache, void* v_cache, const int32_t* slot_mapping,
+                                      int64_t n_rows, int64_t num_q_heads, int64_t num_kv_heads,
+                                      int64_t head_dim, int64_t num_slots,
+                                      int write_k_inplace, void* stream);
+
 /* ------------------------------------------------------------------ 2. paged decode attention
  * Replaces flash_attn_with_kvcache(q[B,1,Hq,D], k_cache, v_cache, cache_seqlens=context_lens,
  * block_table=block_tables, softmax_scale=scale, causal=True) at infer/ops/attention.py:118-120,

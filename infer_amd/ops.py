@@ -55,6 +55,39 @@ def store_kvcache(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor,
     _lib.check(rc, "store_kvcache")
 
 
+def qk_norm_rope_store_kvcache(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, positions: torch.Tensor,
+                               q_norm_weight: torch.Tensor, k_norm_weight: torch.Tensor, eps: float,
+                               cos_sin_cache: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                               slot_mapping: torch.Tensor, write_key: bool = True) -> None:
+    """One launch for ``q_norm``, ``k_norm``, the in-place neox rotary embedding and ``store_kvcache``
+    (the sequence at ``infer/models/Qwen3.py:113-131``).  ``q`` ``[N, Hq, D]`` and ``k`` ``[N, Hkv, D]``
+    are updated in place (``k`` only if ``write_key``), the rotated ``k`` and ``v`` land in the caches
+    at ``slot_mapping``; rows with a negative slot skip the caches."""
+    n, hq, d = q.shape
+    hkv = k.shape[1]
+    assert k.shape == (n, hkv, d) and v.shape == (n, hkv, d)
+    for t in (q, k, v, q_norm_weight, k_norm_weight, cos_sin_cache, k_cache, v_cache):
+        assert t.dtype == torch.bfloat16
+    for t in (q, k, v):
+        assert t.stride(2) == 1 and t.stride(1) == d
+    assert q_norm_weight.shape == (d,) and k_norm_weight.shape == (d,)
+    assert q_norm_weight.is_contiguous() and k_norm_weight.is_contiguous()
+    assert cos_sin_cache.dim() == 2 and cos_sin_cache.shape[1] == d and cos_sin_cache.is_contiguous()
+    assert positions.dtype == torch.int64 and positions.numel() == n and positions.is_contiguous()
+    assert slot_mapping.dtype == torch.int32 and slot_mapping.numel() == n and slot_mapping.is_contiguous()
+    assert k_cache.stride(1) == hkv * d and v_cache.stride(1) == hkv * d
+    assert k_cache.stride(0) == k_cache.shape[1] * hkv * d and v_cache.stride(0) == v_cache.shape[1] * hkv * d
+    _require_gpu(q, k, v, positions, q_norm_weight, k_norm_weight, cos_sin_cache, k_cache, v_cache, slot_mapping)
+    if n == 0:
+        return
+    rc = _lib.load().infer_kv_qk_norm_rope_append_bf16(
+        q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), positions.data_ptr(),
+        q_norm_weight.data_ptr(), k_norm_weight.data_ptr(), float(eps), cos_sin_cache.data_ptr(),
+        cos_sin_cache.shape[0], k_cache.data_ptr(), v_cache.data_ptr(), slot_mapping.data_ptr(), n, hq, hkv, d,
+        k_cache.shape[0] * k_cache.shape[1], int(bool(write_key)), _stream_ptr(q))
+    _lib.check(rc, "qk_norm_rope_store_kvcache")
+
+
 def decode_workspace(device, max_batch: int, num_q_heads: int, num_kv_heads: int, head_dim: int) -> torch.Tensor:
     """Workspace for the split-KV partial results, cached per (device, shape): allocated once so that
     steady-state decode steps (and HIP graph replays) never allocate."""
