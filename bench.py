@@ -200,6 +200,22 @@ def main():
     ap_ms = gpu_time_ms(append_step, max(args.steps, 48), reps)
     append_gbs = p3.append_bytes / (ap_ms * 1e-3) / 1e9
 
+    # fused QK-norm + RoPE + append (one launch for the four steps in front of attention)
+    def fused_case(n_rows):
+        d_ = 128
+        qkv = torch.randn((n_rows, (hq + 2 * hkv) * d_), dtype=torch.bfloat16, device=dev)
+        q_, k_, v_ = (t.view(n_rows, -1, d_) for t in qkv.split([hq * d_, hkv * d_, hkv * d_], dim=-1))
+        w_ = torch.ones(d_, dtype=torch.bfloat16, device=dev)
+        cs_ = torch.randn((4096, d_), dtype=torch.bfloat16, device=dev)
+        pos_ = torch.randint(0, 4096, (n_rows,), device=dev)
+        sl_ = torch.randperm(p3.k_cache.shape[0] * 256, device=dev)[:n_rows].to(torch.int32)
+        ms_ = gpu_time_ms(lambda: ops.qk_norm_rope_store_kvcache(q_, k_, v_, pos_, w_, w_, 1e-6, cs_, dsts[0][0],
+                                                                 dsts[0][1], sl_), 50, 5)
+        nbytes_ = n_rows * (2 * hq * d_ * 2 + 5 * hkv * d_ * 2)   # q r+w, k r+w+cache, v r+cache
+        return round(ms_ * 1e3, 2), round(nbytes_ / ms_ / 1e6, 1)
+    fused_small = fused_case(b)
+    fused_big = fused_case(int(p3.q.shape[0]))
+
     # paged varlen causal prefill attention on the same cfg3 step (after its append), for the record
     kc3, vc3 = p3.k_cache.clone(), p3.v_cache.clone()
     ops.store_kvcache(p3.k_new, p3.v_new, kc3, vc3, p3.slot_mapping)
@@ -231,6 +247,11 @@ def main():
     line["prefill_attention"] = {"workload": "cfg3: 16 prompts U[64,2048], 0-50 % cached, causal over the paged cache",
                                  "query_tokens": int(p3.q.shape[0]), "ms": round(pf_ms, 4),
                                  "TFLOPs": round(pf_flops / (pf_ms * 1e-3) / 1e12, 1)}
+    line["fused_qk_norm_rope_append"] = {"decode_rows": b, "decode_us": fused_small[0],
+                                         "prefill_rows": int(p3.q.shape[0]), "prefill_us": fused_big[0],
+                                         "prefill_GBps": fused_big[1],
+                                         "note": "same 161 MB qkv buffer every launch: partly served by the "
+                                                 "256 MB Infinity Cache, not an HBM figure"}
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline()
     print(json.dumps(line))
