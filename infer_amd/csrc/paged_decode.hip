@@ -582,16 +582,24 @@ __global__ void __launch_bounds__(256) paged_decode_merge_kernel(MergeArgs a) {
 
 int g_split_workgroups = 0;
 
+constexpr int kMaxDevices = 64;
+
+int current_device() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+    return dev;
+}
+
+// Compute units of the current device (cached per device; a benign race writes the same value).
 int device_cu_count() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess) return 256;
+    static int cus[kMaxDevices] = {0};
+    const int dev = current_device();
+    if (cus[dev] == 0) {
         int v = 0;
         if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) return 256;
-        cus = v;
+        cus[dev] = v;
     }
-    return cus;
+    return cus[dev];
 }
 
 struct Launch {
@@ -692,12 +700,13 @@ int infer_paged_decode_split_bf16(const void* q, int64_t q_stride0, const void* 
     a.slots_per_head = L.W + (int)batch;
 
     const size_t lds_bytes = (size_t)L.waves * kLdsPerWave;
-    static bool attr_set = false;
-    if (!attr_set) {
+    static bool attr_set[kMaxDevices] = {false};   // the attribute is per device
+    const int dev = current_device();
+    if (!attr_set[dev]) {
         hipError_t e = hipFuncSetAttribute((const void*)paged_decode_split_kernel,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 8 * kLdsPerWave);
         if (e != hipSuccess) return (int)e;
-        attr_set = true;
+        attr_set[dev] = true;
     }
     dim3 grid(L.W, L.grid_y, 1), block(64 * L.waves, 1, 1);
     hipLaunchKernelGGL(paged_decode_split_kernel, grid, block, lds_bytes, (hipStream_t)stream, a);

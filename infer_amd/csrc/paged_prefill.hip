@@ -501,12 +501,14 @@ extern "C" int infer_paged_prefill_bf16(const void* q, int64_t q_stride0, const 
         default: break;
     }
     const size_t lds_bytes = (size_t)G * kLdsWave;
-    static bool attr_set = false;
-    if (!attr_set) {
+    static bool attr_set[64] = {false};   // the attribute is per device
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    if (!attr_set[dev]) {
         hipError_t e = hipFuncSetAttribute((const void*)paged_prefill_kernel,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 16 * kLdsWave);
         if (e != hipSuccess) return (int)e;
-        attr_set = true;
+        attr_set[dev] = true;
     }
     dim3 grid((unsigned)((max_seqlen_q + kQTile - 1) / kQTile), (unsigned)num_seqs, (unsigned)num_kv_heads);
     dim3 block(64 * G, 1, 1);
