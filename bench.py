@@ -70,6 +70,44 @@ def cpu_baseline(sample_seqs=16, min_seconds=10.0):
     }
 
 
+def run_e2e(args):
+    """End-to-end decode through the engine: random-init model of a published Qwen3 shape, batch of
+    random-token prompts with lengths uniform in [128, 1024], greedy decoding, KV pool filling the
+    free HBM, decode step replayed as a HIP graph.  Prints one JSON line."""
+    import numpy as np
+    from infer_amd import config as C
+    from infer_amd.llm_engine import LLMEngine
+    from infer_amd.sampling_params import SamplingParams
+    hf = {"8b": C.qwen3_8b, "0.6b": C.qwen3_0_6b, "32b": C.qwen3_32b}[args.e2e_model]()
+    t0 = time.perf_counter()
+    engine = LLMEngine(hf_config=hf, max_num_seqs=max(args.e2e_batch, 16), max_model_len=4096,
+                       max_num_batched_tokens=16384, enforce_eager=args.e2e_eager, seed=0)
+    torch.cuda.synchronize()
+    t_init = time.perf_counter() - t0
+    rng = np.random.default_rng(0)
+    lengths = rng.integers(128, 1025, size=args.e2e_batch)
+    prompts = [[int(t) for t in rng.integers(0, hf.vocab_size, size=int(n))] for n in lengths]
+    sp = SamplingParams(temperature=0.0, max_tokens=args.e2e_new, ignore_eos=True)
+    t0 = time.perf_counter()
+    outs = engine.generate(prompts, sp)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    st = engine.stats
+    assert all(len(o["token_ids"]) == args.e2e_new for o in outs)
+    dec_tps = st["decode_tokens"] / st["decode_s"] if st["decode_s"] else 0.0
+    print(json.dumps({
+        "metric": "end-to-end greedy decode throughput through the engine", "value": round(dec_tps, 1),
+        "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"cfg5: random-init Qwen3-{args.e2e_model} decode, batch {args.e2e_batch}, prompts "
+                               f"U[128,1024], {args.e2e_new} greedy tokens, hipGraph={not args.e2e_eager}"},
+        "decode_steps": st["decode_steps"], "decode_ms_per_step": round(1e3 * st["decode_s"] / max(st["decode_steps"], 1), 3),
+        "prefill_tokens_per_s": round(st["prefill_tokens"] / st["prefill_s"], 1) if st["prefill_s"] else None,
+        "prefill_steps": st["prefill_steps"], "generate_wall_s": round(wall, 2), "init_s": round(t_init, 1),
+        "num_kvcache_blocks": engine.config.num_kvcache_blocks,
+        "kv_pool_GB": round(engine.model_runner.kv_cache.numel() * 2 / 1e9, 1),
+        "graphs": len(engine.model_runner.graphs)}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -84,6 +122,13 @@ def main():
     ap.add_argument("--counters", action="store_true",
                     help="short untimed run for `rocprofv3 --pmc`: a 1 GiB plain copy (x3), the decode op (x5), "
                          "a prefill-sized append (x3)")
+    ap.add_argument("--e2e", action="store_true",
+                    help="end-to-end decode through the engine (random-init Qwen3, HIP-graph decode) instead "
+                         "of the kernel benchmark")
+    ap.add_argument("--e2e-model", default="8b", choices=["0.6b", "8b", "32b"])
+    ap.add_argument("--e2e-batch", type=int, default=128)
+    ap.add_argument("--e2e-new", type=int, default=256)
+    ap.add_argument("--e2e-eager", action="store_true", help="run the decode steps eagerly (no HIP graph)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this path needs no collective and every box here has one GPU; "
@@ -93,6 +138,9 @@ def main():
         print("bench.py needs a GPU: the HIP kernels are the only implementation of the path", file=sys.stderr)
         sys.exit(2)
 
+    if args.e2e:
+        run_e2e(args)
+        return
     from infer_amd import ops, workloads
     dev = torch.device("cuda:0")
     if args.ceiling:

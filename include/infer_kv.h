@@ -183,6 +183,37 @@ int infer_paged_prefill_bf16(const void* q, int64_t q_stride0,
  * (0 = choose from the device's CU count).  Process-wide; returns the previous value. */
 int infer_paged_decode_set_split_workgroups(int workgroups);
 
+/* ------------------------------------------------------------------ 2c. the operators of a decode step around the path
+ * What the engine runs between two attention calls of a captured decode step, so that the step is
+ * HIP kernels of this library plus library GEMMs.
+ *
+ * infer_rms_norm_bf16 replaces RMSNorm.forward (infer/ops/norm.py:63-98; the torch path the engine
+ * runs, rms_forward / add_rms_forward).  Without residual: out = bf16(x * rsqrt(mean(x^2) + eps)) *
+ * weight.  With residual: s = float(x) + float(residual); residual <- bf16(s); out from the
+ * unrounded s.  out may alias x.  Rows are [n_rows, hidden] bf16 with the given row strides
+ * (elements); hidden % 8 == 0 and hidden <= 8192.
+ */
+int infer_rms_norm_bf16(const void* x, int64_t x_stride0, void* residual, int64_t residual_stride0,
+                        const void* weight, void* out, int64_t out_stride0,
+                        int64_t n_rows, int64_t hidden, float eps, void* stream);
+
+/* Replaces silu_and_mul(result, input) (src/operators/silu/silu.cu:13-54; schema src/bindings.cpp:22):
+ * out[r, j] = bf16(silu(x[r, j])) * x[r, d + j] for x [n_rows, 2 d] bf16, d % 8 == 0. */
+int infer_silu_and_mul_bf16(void* out, int64_t out_stride0, const void* x, int64_t x_stride0,
+                            int64_t n_rows, int64_t d, void* stream);
+
+/* Replaces the host loop of ModelRunner.prepare_decode (infer/engine/model_runner.py:110-126) by
+ * one launch on device-resident state.  seq_lens[b] = len(seq) including the token fed this step:
+ *   context_lens[b] = len, positions[b] = len - 1 + position_offset,
+ *   slot_mapping[b] = block_table[b, (len-1) / block_size] * block_size + (len-1) % block_size.
+ * position_offset = 1 reproduces the reference (model_runner.py:117 feeds len(seq)); 0 gives the
+ * zero-based position of its prefill branch (:84).  Rows with seq_lens[b] <= 0 (graph padding) get
+ * slot -1, context length 0 and position 0, so they neither touch the cache nor attend. */
+int infer_decode_metadata(const int32_t* seq_lens, const int32_t* block_table, int64_t bt_stride0,
+                          int64_t batch, int64_t block_size, int64_t table_cols,
+                          int64_t position_offset, int64_t* positions, int32_t* slot_mapping,
+                          int32_t* context_lens, void* stream);
+
 /* ------------------------------------------------------------------ measurement helpers
  * No counterpart in the reference.  Plain streaming kernels used by bench.py --ceiling to measure
  * what the part sustains for a read-only stream (same launch shape as the decode kernel: one
@@ -223,6 +254,11 @@ int infer_pool_can_append(const infer_pool* pool, int64_t seq_len);
  * to `table` (capacity must allow num_blocks + 1 then).  Returns the new number of blocks. */
 int64_t infer_pool_may_append(infer_pool* pool, const int64_t* token_ids, int64_t seq_len,
                               int32_t* table, int64_t num_blocks, int64_t table_capacity);
+/* The same step given only the block_size tokens of the block that seq_len just filled (read only
+ * when seq_len % block_size == 0, may be NULL otherwise), so a per-token caller does not have to
+ * hand over the whole sequence. */
+int64_t infer_pool_may_append_block(infer_pool* pool, const int64_t* last_block_tokens, int64_t seq_len,
+                                    int32_t* table, int64_t num_blocks, int64_t table_capacity);
 
 /* compute_hash :54-60: xxh64(seed 0) over [prefix hash as 8 LE bytes, if has_prefix] ++ int64 LE ids. */
 uint64_t infer_pool_hash(const int64_t* token_ids, int64_t n, int has_prefix, uint64_t prefix_hash);

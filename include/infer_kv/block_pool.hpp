@@ -56,6 +56,9 @@ public:
     // opens a new block when the new token is the first of a block, seals (hashes and registers)
     // the last block when the new token filled it.
     void may_append(const int64_t* token_ids, int64_t seq_len, std::vector<int32_t>& table);
+    // Same, for callers that keep only the tail of a long sequence at hand: `last_block_tokens` are the
+    // block_size tokens of the block that seq_len just filled (read only when seq_len % block_size == 0).
+    void may_append_block(const int64_t* last_block_tokens, int64_t seq_len, std::vector<int32_t>& table);
 
     // Raw allocation without token ids (no prefix sharing), for callers that only know lengths:
     // takes the block at the front of the free FIFO / drops one reference.

@@ -35,6 +35,9 @@ SIGNATURES = {
     "infer_paged_decode_set_split_workgroups": (_c.c_int, [_c.c_int]),
     "infer_paged_prefill_bf16": (_c.c_int, [_vp, _i64, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _i64,
                                             _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _c.c_int, _vp]),
+    "infer_rms_norm_bf16": (_c.c_int, [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _f32, _vp]),
+    "infer_silu_and_mul_bf16": (_c.c_int, [_vp, _i64, _vp, _i64, _i64, _i64, _vp]),
+    "infer_decode_metadata": (_c.c_int, [_vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
     "infer_kv_probe_read": (_c.c_int, [_vp, _sz, _vp, _c.c_int, _vp]),
     "infer_kv_probe_copy": (_c.c_int, [_vp, _vp, _sz, _c.c_int, _vp]),
     "infer_pool_create": (_vp, [_i32, _i32]),
@@ -47,6 +50,7 @@ SIGNATURES = {
     "infer_pool_deallocate": (_c.c_int, [_vp, _vp, _i64]),
     "infer_pool_can_append": (_c.c_int, [_vp, _i64]),
     "infer_pool_may_append": (_i64, [_vp, _vp, _i64, _vp, _i64, _i64]),
+    "infer_pool_may_append_block": (_i64, [_vp, _vp, _i64, _vp, _i64, _i64]),
     "infer_pool_hash": (_c.c_uint64, [_vp, _i64, _c.c_int, _c.c_uint64]),
     "infer_xxh64": (_c.c_uint64, [_vp, _sz, _c.c_uint64]),
     "infer_pool_ref_count": (_i32, [_vp, _i32]),

@@ -24,13 +24,15 @@ class Attention(torch.nn.Module):
         self.num_kv_heads = num_kv_heads
         self.k_cache = self.v_cache = torch.tensor([])
 
-    def forward(self, Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor) -> torch.Tensor:
+    def forward(self, Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, kv_stored: bool = False) -> torch.Tensor:
+        """``kv_stored`` says that the caller has already written ``K``/``V`` to the caches (the fused
+        norm + rotary + append kernel does), so the append of ``attention.py:108-109`` is skipped."""
         Q = Q.view(-1, self.num_heads, self.head_dim)
         K = K.view(-1, self.num_kv_heads, self.head_dim)
         V = V.view(-1, self.num_kv_heads, self.head_dim)
         context = get_context()
         k_cache, v_cache = self.k_cache, self.v_cache
-        if k_cache.numel() and v_cache.numel():
+        if k_cache.numel() and v_cache.numel() and not kv_stored:
             ops.store_kvcache(K, V, k_cache, v_cache, context.slot_mapping)
         if context.is_prefill:
             if context.block_tables is not None:   # prefix cache: keys come from the paged cache

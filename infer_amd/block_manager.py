@@ -93,11 +93,15 @@ class BlockManager:
         return bool(self._lib.infer_pool_can_append(self._pool, len(seq)))
 
     def may_append(self, seq: Sequence):
-        ids = self._ids(seq.token_ids)
+        r = len(seq) % self.block_size
+        if r > 1 and seq.block_table:
+            return           # mid-block token: the reference only asserts here (``:132-133``)
+        # only the block that was just filled has to cross the boundary, not the whole sequence
+        ids = self._ids(seq.token_ids[-self.block_size:]) if r == 0 else None
         n = len(seq.block_table)
         table = np.empty(n + 1, dtype=np.int32)
         table[:n] = seq.block_table
-        new_n = self._state(self._lib.infer_pool_may_append(self._pool, ids.ctypes.data, ids.size,
-                                                            table.ctypes.data, n, table.size))
+        new_n = self._state(self._lib.infer_pool_may_append_block(
+            self._pool, ids.ctypes.data if ids is not None else None, len(seq), table.ctypes.data, n, table.size))
         if new_n > n:
             seq.block_table.append(int(table[n]))

@@ -206,6 +206,12 @@ bool BlockPool::can_append(int64_t seq_len) const {
 }
 
 void BlockPool::may_append(const int64_t* token_ids, int64_t seq_len, std::vector<int32_t>& table) {
+    const int64_t full = seq_len / block_size_;
+    const bool seals = seq_len > 0 && seq_len % block_size_ == 0;
+    may_append_block(seals ? token_ids + (full - 1) * block_size_ : nullptr, seq_len, table);
+}
+
+void BlockPool::may_append_block(const int64_t* blk_tokens, int64_t seq_len, std::vector<int32_t>& table) {
     std::lock_guard<std::mutex> g(mu_);
     if (table.empty()) throw std::logic_error("BlockPool::may_append: sequence holds no blocks");
     Block& last = blocks_[table.back()];
@@ -218,8 +224,7 @@ void BlockPool::may_append(const int64_t* token_ids, int64_t seq_len, std::vecto
         table.push_back(id);
     } else if (r == 0) {
         if (last.hashed) throw std::logic_error("BlockPool::may_append: block sealed twice");
-        const int64_t nblocks = seq_len / block_size_;
-        const int64_t* blk_tokens = token_ids + (nblocks - 1) * block_size_;
+        if (!blk_tokens) throw std::logic_error("BlockPool::may_append: tokens of the block to seal are missing");
         const bool has_prev = table.size() > 1;
         const Block* prev = has_prev ? &blocks_[table[table.size() - 2]] : nullptr;
         // the reference passes the previous block's hash, or -1 when there is none (or it is unsealed)
@@ -339,6 +344,20 @@ int64_t infer_pool_may_append(infer_pool* p, const int64_t* token_ids, int64_t s
     return guarded([&]() -> int64_t {
         std::vector<int32_t> t(table, table + num_blocks);
         p->pool.may_append(token_ids, seq_len, t);
+        for (size_t i = 0; i < t.size(); ++i) table[i] = t[i];
+        return static_cast<int64_t>(t.size());
+    });
+}
+
+int64_t infer_pool_may_append_block(infer_pool* p, const int64_t* last_block_tokens, int64_t seq_len, int32_t* table,
+                                    int64_t num_blocks, int64_t table_capacity) {
+    if (!p || !table || seq_len <= 0 || num_blocks <= 0 || table_capacity < num_blocks) return INFER_KV_EINVAL;
+    const int64_t r = seq_len % p->pool.block_size();
+    if (r == 1 && table_capacity < num_blocks + 1) return INFER_KV_EINVAL;
+    if (r == 0 && !last_block_tokens) return INFER_KV_EINVAL;
+    return guarded([&]() -> int64_t {
+        std::vector<int32_t> t(table, table + num_blocks);
+        p->pool.may_append_block(last_block_tokens, seq_len, t);
         for (size_t i = 0; i < t.size(); ++i) table[i] = t[i];
         return static_cast<int64_t>(t.size());
     });

@@ -16,6 +16,7 @@ import torch
 from . import _lib
 
 _workspaces: dict = {}
+_retired_workspaces: list = []      # outgrown workspaces stay alive: captured graphs may still point at them
 
 
 def _stream_ptr(t: torch.Tensor) -> int:
@@ -99,6 +100,8 @@ def decode_workspace(device, max_batch: int, num_q_heads: int, num_kv_heads: int
         if nbytes == 0:
             raise RuntimeError("paged decode: unsupported shape "
                                f"(Hq={num_q_heads}, Hkv={num_kv_heads}, D={head_dim})")
+        if ws is not None:
+            _retired_workspaces.append(ws[1])
         ws = (cap, torch.empty(nbytes, dtype=torch.uint8, device=device))
         _workspaces[key] = ws
     return ws[1]
@@ -216,6 +219,64 @@ def flash_attn_varlen_func(q, k, v, *, max_seqlen_q, cu_seqlens_q, max_seqlen_k,
         nseq, int(max_seqlen_q), hq, hkv, d, bs, nblk, float(softmax_scale), int(bool(causal)), _stream_ptr(q))
     _lib.check(rc, "flash_attn_varlen_func")
     return out
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.Tensor | None = None,
+             out: torch.Tensor | None = None):
+    """``RMSNorm.forward`` of ``infer/ops/norm.py:63-98``: returns ``out`` or, with ``residual``,
+    ``(out, residual)`` where ``residual`` has been updated in place to ``x + residual``."""
+    hidden = x.shape[-1]
+    x2 = x.reshape(-1, hidden)
+    assert x2.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x2.stride(1) == 1
+    assert weight.shape == (hidden,) and weight.is_contiguous()
+    if out is None:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    o2 = out.view(-1, hidden)
+    assert o2.shape == x2.shape and o2.dtype == torch.bfloat16 and o2.stride(1) == 1
+    r2 = None
+    if residual is not None:
+        r2 = residual.view(-1, hidden)
+        assert r2.shape == x2.shape and r2.dtype == torch.bfloat16 and r2.stride(1) == 1
+    _require_gpu(x2, weight, o2, *([r2] if r2 is not None else []))
+    rc = _lib.load().infer_rms_norm_bf16(
+        x2.data_ptr(), x2.stride(0), r2.data_ptr() if r2 is not None else None,
+        r2.stride(0) if r2 is not None else 0, weight.data_ptr(), o2.data_ptr(), o2.stride(0),
+        x2.shape[0], hidden, float(eps), _stream_ptr(x))
+    _lib.check(rc, "rms_norm")
+    return out if residual is None else (out, residual)
+
+
+def silu_and_mul(out: torch.Tensor, x: torch.Tensor) -> None:
+    """``silu_and_mul(result, input)`` of ``src/bindings.cpp:22``: ``out = silu(x[..., :d]) * x[..., d:]``."""
+    d = x.shape[-1] // 2
+    x2 = x.reshape(-1, 2 * d)
+    o2 = out.view(-1, d)
+    assert x.shape[-1] == 2 * d and o2.shape[0] == x2.shape[0]
+    assert x2.dtype == torch.bfloat16 and o2.dtype == torch.bfloat16 and x2.stride(1) == 1 and o2.stride(1) == 1
+    _require_gpu(x2, o2)
+    rc = _lib.load().infer_silu_and_mul_bf16(o2.data_ptr(), o2.stride(0), x2.data_ptr(), x2.stride(0),
+                                             x2.shape[0], d, _stream_ptr(x))
+    _lib.check(rc, "silu_and_mul")
+
+
+def decode_metadata(seq_lens: torch.Tensor, block_table: torch.Tensor, block_size: int, position_offset: int,
+                    positions: torch.Tensor, slot_mapping: torch.Tensor, context_lens: torch.Tensor) -> None:
+    """Derives a decode step's ``positions`` / ``slot_mapping`` / ``context_lens`` on the device from
+    the sequence lengths and the block table (``infer/engine/model_runner.py:110-126``); rows with
+    length 0 are padding (slot -1, context length 0)."""
+    b = seq_lens.numel()
+    assert seq_lens.dtype == torch.int32 and seq_lens.is_contiguous()
+    assert block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.shape[0] == b
+    assert block_table.stride(1) == 1
+    assert positions.dtype == torch.int64 and slot_mapping.dtype == torch.int32 and context_lens.dtype == torch.int32
+    for t in (positions, slot_mapping, context_lens):
+        assert t.numel() == b and t.is_contiguous()
+    _require_gpu(seq_lens, block_table, positions, slot_mapping, context_lens)
+    rc = _lib.load().infer_decode_metadata(
+        seq_lens.data_ptr(), block_table.data_ptr(), block_table.stride(0), b, int(block_size),
+        block_table.shape[1], int(position_offset), positions.data_ptr(), slot_mapping.data_ptr(),
+        context_lens.data_ptr(), _stream_ptr(seq_lens))
+    _lib.check(rc, "decode_metadata")
 
 
 def set_split_workgroups(n: int) -> int:

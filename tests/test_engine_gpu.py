@@ -1,0 +1,169 @@
+"""The engine end to end on the GPU (scheduler -> model runner -> fused front end -> paged attention ->
+sampler) on a tiny random Qwen3, against ``oracle/qwen3_ref.py`` (float32, dense attention over the
+whole sequence, pinned against the ``transformers`` implementation on the CPU).
+
+Bar: logits of every step within ``LOGIT_TOL`` (relative to the largest logit of the row; the model
+computes in bf16, the oracle in float32); the token the engine picks is within that tolerance of the
+oracle's best token; a HIP-graph replay is bit-identical to the eager step on the same inputs."""
+import numpy as np
+import pytest
+import torch
+
+from infer_amd.config import Config, ModelConfig
+from infer_amd.context import reset_context
+from infer_amd.sampling_params import SamplingParams
+from oracle import qwen3_ref
+
+pytestmark = pytest.mark.gpu
+
+TINY = dict(vocab_size=512, hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+            num_key_value_heads=2, head_dim=128, max_position_embeddings=2048, rope_theta=1e6, rms_norm_eps=1e-6,
+            tie_word_embeddings=False)
+LOGIT_TOL = 4e-2
+
+
+def make_config(**kw):
+    base = dict(hf_config=ModelConfig(**TINY), num_kvcache_blocks=24, max_model_len=2048,
+                max_num_batched_tokens=4096, max_num_seqs=16, enforce_eager=True, seed=11)
+    base.update(kw)
+    return Config(**base)
+
+
+def prompts(lengths, seed=0):
+    g = np.random.default_rng(seed)
+    return [[int(t) for t in g.integers(0, TINY["vocab_size"], size=n)] for n in lengths]
+
+
+def oracle_logits(runner, seq, offset):
+    """Oracle logits for the newest token of ``seq``, from the engine's weights, its rotary table and the
+    positions it feeds."""
+    from infer_amd.layers import cos_sin_table
+    cfg = runner.config.hf_config
+    table = cos_sin_table(cfg.head_dim, cfg.max_position_embeddings, cfg.rope_theta, runner.device)
+    pos = qwen3_ref.engine_positions(seq.num_prompt_tokens, len(seq), offset)
+    return qwen3_ref.forward_full(dict(runner.model.named_parameters()), cfg, seq.token_ids, pos, table)[-1]
+
+
+def check_step(runner, seqs, logits, offset):
+    picked = logits.float().argmax(dim=-1).tolist()
+    for seq, row, tok in zip(seqs, logits.float().cpu(), picked):
+        want = oracle_logits(runner, seq, offset)
+        scale = want.abs().max().item()
+        assert torch.isfinite(row).all()
+        assert (row - want).abs().max().item() <= LOGIT_TOL * scale, (len(seq), (row - want).abs().max().item(), scale)
+        assert want.max().item() - want[tok].item() <= 2 * LOGIT_TOL * scale
+    return picked
+
+
+@pytest.mark.parametrize("offset", [1, 0])
+def test_prefill_then_decode_steps_match_oracle(gpu, offset):
+    from infer_amd.model_runner import ModelRunner
+    from infer_amd.scheduler import Scheduler
+    from infer_amd.sequence import Sequence
+    config = make_config(decode_position_offset=offset)
+    runner = ModelRunner(config)
+    sched = Scheduler(config)
+    for p in prompts([5, 300, 517]):
+        sched.add(Sequence(p, SamplingParams(0.0, 6, True)))
+    steps = 0
+    while not sched.is_finished():
+        seqs, is_prefill = sched.schedule()
+        assert is_prefill == (steps == 0)
+        logits = runner.run_model(seqs, is_prefill)
+        reset_context()
+        tokens = check_step(runner, seqs, logits, offset)
+        sched.postprocess(seqs, tokens)
+        steps += 1
+    assert steps == 6
+
+
+def test_graph_replay_is_bit_identical_to_eager_and_padding_rows_touch_nothing(gpu):
+    from infer_amd.model_runner import ModelRunner
+    from infer_amd.scheduler import Scheduler
+    from infer_amd.sequence import Sequence
+    config = make_config(enforce_eager=False, max_num_seqs=16)
+    runner = ModelRunner(config)
+    assert runner.graph_bs == [1, 2, 4, 8, 16] and set(runner.graphs) == set(runner.graph_bs)
+    sched = Scheduler(config)
+    seqs = [Sequence(p, SamplingParams(0.0, 8, True)) for p in prompts([40, 255, 256], seed=3)]
+    for s in seqs:
+        sched.add(s)
+    batch, is_prefill = sched.schedule()
+    sched.postprocess(batch, runner.run(batch, is_prefill))
+    owned = {b for s in seqs for b in s.block_table}
+    runner.kv_cache[:, :, [b for b in range(config.num_kvcache_blocks) if b not in owned]] = 77.0
+    for step in range(5):
+        batch, is_prefill = sched.schedule()
+        assert not is_prefill and len(batch) == 3
+        owned |= {b for s in seqs for b in s.block_table}
+        run_bs = runner.prepare_decode(batch)
+        assert run_bs == 4                                   # three sequences ride the graph of four
+        with torch.inference_mode():
+            eager = runner._decode_forward(run_bs).clone()
+            reset_context()
+            torch.cuda.synchronize()
+            runner.graphs[run_bs].replay()
+            torch.cuda.synchronize()
+            replay = runner.d_outputs[:run_bs].clone()
+            assert torch.equal(eager[:3], replay[:3]), f"replay {step} differs from eager"
+            logits = runner.model.compute_logits(replay[:3])
+        tokens = check_step(runner, batch, logits, config.decode_position_offset)
+        sched.postprocess(batch, tokens)
+    free = [b for b in range(config.num_kvcache_blocks) if b not in owned]
+    assert (runner.kv_cache[:, :, free] == 77.0).all()       # the padding row wrote to no block
+
+
+def test_generate_graph_and_eager_agree_and_prefix_cache_hits(gpu):
+    from infer_amd.llm_engine import LLMEngine
+    ps = prompts([30, 130, 260, 511], seed=5)
+    sp = SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True)
+    kw = dict(hf_config=ModelConfig(**TINY), num_kvcache_blocks=24, max_model_len=2048,
+              max_num_batched_tokens=4096, max_num_seqs=16, seed=11)
+    eager = LLMEngine(enforce_eager=True, **kw)
+    graph = LLMEngine(enforce_eager=False, **kw)
+    out_e = eager.generate(ps, sp)
+    out_g = graph.generate(ps, sp)
+    assert [o["token_ids"] for o in out_e] == [o["token_ids"] for o in out_g]
+    assert all(len(o["token_ids"]) == 12 for o in out_g)
+    assert graph.stats["decode_steps"] == 11 and graph.stats["prefill_steps"] == 1
+    assert graph.scheduler.block_manager.num_free_blocks == 24
+
+    # a second request that shares the first 256 tokens of prompt 3 finds that block in the cache
+    from infer_amd.sequence import Sequence
+    again = ps[3][:256] + prompts([100], seed=9)[0]
+    seq = Sequence(again, SamplingParams(0.0, 3, True))
+    graph.scheduler.add(seq)
+    batch, is_prefill = graph.scheduler.schedule()
+    assert is_prefill and seq.num_cached_tokens == 256
+    logits = graph.model_runner.run_model(batch, True)
+    reset_context()
+    tokens = check_step(graph.model_runner, batch, logits, graph.config.decode_position_offset)
+    graph.scheduler.postprocess(batch, tokens)
+    while not graph.is_finished():
+        graph.step()
+    assert seq.num_completion_tokens == 3
+
+
+def test_preemption_under_a_tiny_pool_still_finishes(gpu):
+    from infer_amd.llm_engine import LLMEngine
+    engine = LLMEngine(hf_config=ModelConfig(**TINY), num_kvcache_blocks=4, max_model_len=2048,
+                       max_num_batched_tokens=4096, max_num_seqs=8, enforce_eager=False, seed=11)
+    ps = prompts([250, 251, 252], seed=7)
+    outs = engine.generate(ps, SamplingParams(0.0, 10, True))
+    assert [len(o["token_ids"]) for o in outs] == [10, 10, 10]
+    assert engine.stats["prefill_steps"] > 1                 # somebody was evicted and prefetched again
+    assert engine.scheduler.block_manager.num_free_blocks == 4
+
+
+def test_sampler_temperature(gpu):
+    from infer_amd.layers import Sampler
+    torch.manual_seed(0)
+    logits = torch.full((4, 100), -20.0, device=gpu, dtype=torch.bfloat16)
+    logits[:, 7] = 20.0
+    temps = torch.tensor([0.0, 1.0, 0.5, 0.0], device=gpu)
+    assert Sampler()(logits, temps).tolist() == [7, 7, 7, 7]
+    assert Sampler()(logits, temps * 0, all_greedy=True).tolist() == [7, 7, 7, 7]
+    flat = torch.zeros((2000, 4), device=gpu)
+    draws = Sampler()(flat, torch.ones(2000, device=gpu))
+    counts = torch.bincount(draws, minlength=4).float() / 2000
+    assert (counts - 0.25).abs().max() < 0.05                # uniform logits: every token about equally often
