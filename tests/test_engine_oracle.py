@@ -171,3 +171,36 @@ def test_sequence_wire_form_roundtrip():
     s.append_token(8)
     t = pickle.loads(pickle.dumps(s))
     assert t.last_token == 8 and t.num_tokens == 4 and not hasattr(t, "token_ids")
+
+
+def test_weight_loader_maps_a_checkpoint_onto_the_packed_parameters(tmp_path):
+    """A checkpoint in the published tensor naming (separate q/k/v and gate/up projections), written
+    by the ``transformers`` model, must land in the engine's packed parameters so that the oracle on
+    the loaded weights reproduces the ``transformers`` logits."""
+    from safetensors.torch import save_file
+    from infer_amd.qwen3 import QwenForCausalLM
+    from infer_amd.weight_loader import has_checkpoint, load_model
+    model = _hf_model()
+    assert not has_checkpoint(str(tmp_path))
+    state = {k: v.to(torch.bfloat16).contiguous() for k, v in model.state_dict().items()}
+    names = sorted(state)
+    save_file({k: state[k] for k in names[::2]}, str(tmp_path / "model-00001-of-00002.safetensors"))
+    save_file({k: state[k] for k in names[1::2]}, str(tmp_path / "model-00002-of-00002.safetensors"))
+    (tmp_path / "config.json").write_text(__import__("json").dumps({**TINY, "torch_dtype": "bfloat16"}))
+    assert has_checkpoint(str(tmp_path))
+    cfg = Config(model=str(tmp_path), max_model_len=2048)
+    assert cfg.hf_config.num_key_value_heads == 2 and cfg.hf_config.torch_dtype == torch.bfloat16
+    engine_model = QwenForCausalLM(cfg.hf_config)
+    assert load_model(engine_model, str(tmp_path)) == len(state)
+    want = _packed(state)
+    got = dict(engine_model.named_parameters())
+    assert set(got) == set(want)
+    for name in want:
+        assert torch.equal(got[name].data, want[name]), name
+    tokens = torch.randint(0, TINY["vocab_size"], (9,), generator=torch.Generator().manual_seed(8))
+    model_bf = _hf_model()                                      # same rounded weights on both sides
+    model_bf.load_state_dict({k: v.float() for k, v in state.items()})
+    with torch.no_grad():
+        ref = model_bf(tokens[None]).logits[0]
+    mine = qwen3_ref.forward_full(got, cfg.hf_config, tokens, list(range(9)))
+    assert torch.allclose(mine, ref, atol=1e-4, rtol=1e-4)
