@@ -13,12 +13,19 @@ struct DecodeWorkspace {
     size_t header_off;      // int32[64]: {workgroups, steps per span, total steps}
     size_t seg_first_off;   // int32[batch]: first split workgroup that touched the sequence
     size_t seg_last_off;    // int32[batch]: last one
-    size_t ml_off;          // float[slots][group][2]: running max (log2 domain) and sum
-    size_t po_off;          // float[slots][group][128]: unnormalised accumulator
+    size_t rec_off;         // [slots] records of rec_stride bytes, one per (segment, KV head)
+    size_t rec_stride;      // bytes per record, a multiple of 16
     size_t total_bytes;
 };
 
 static inline size_t align_up_256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+// A partial-result record is written by one wavefront exactly as it sits in that wavefront's
+// registers, so that the store is one contiguous run: for the `group` query heads n of a KV head,
+//   float[4][group][8][4]  accumulator: element (g, n, t, e) is O[n][16 t + 4 g + e] (unnormalised)
+//   float[group][2]        running max (log2 domain) and sum of head n
+// padded to a multiple of 16 bytes.
+static inline size_t decode_record_bytes(int64_t group) { return ((size_t)group * 520 + 15) & ~(size_t)15; }
 
 // slots = num_kv_heads * (INFER_KV_MAX_SPLIT_WG + batch): segment (workgroup w, sequence b) of KV
 // head h uses slot h * (W + batch) + w + b, which is unique because consecutive segments along
@@ -30,8 +37,8 @@ static inline DecodeWorkspace decode_workspace_layout(int64_t batch, int64_t gro
     ws.header_off = off;      off = align_up_256(off + 64 * sizeof(int32_t));
     ws.seg_first_off = off;   off = align_up_256(off + (size_t)batch * sizeof(int32_t));
     ws.seg_last_off = off;    off = align_up_256(off + (size_t)batch * sizeof(int32_t));
-    ws.ml_off = off;          off = align_up_256(off + slots * (size_t)group * 2 * sizeof(float));
-    ws.po_off = off;          off = align_up_256(off + slots * (size_t)group * 128 * sizeof(float));
+    ws.rec_stride = decode_record_bytes(group);
+    ws.rec_off = off;         off = align_up_256(off + slots * ws.rec_stride);
     ws.total_bytes = off;
     return ws;
 }

@@ -66,8 +66,8 @@ struct DecodeArgs {
     int32_t* header;
     int32_t* seg_first;
     int32_t* seg_last;
-    float* ml;          // [slots][group][2]
-    float* po;          // [slots][group][128]
+    unsigned char* rec; // [slots] partial-result records (layout: decode_record_bytes)
+    int rec_stride;
     int slots_per_head; // gridDim.x + batch
 };
 
@@ -256,7 +256,7 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
 
     // Partial results: parked in LDS (lane-private layout, valid lanes only), written out by drain().
     unsigned char* defer = lds + kLdsWave + kPlanBytes;
-    const int slot_bytes = 520 * G;                 // 4G lanes x 8 x 16 B accumulators + G x 8 B (max, sum)
+    const int slot_bytes = a.rec_stride;            // 4G lanes x 8 x 16 B accumulators + G x 8 B (max, sum), padded
     const int defer_cap = kDeferBytes / slot_bytes; // >= 1 for G <= 16
     int ndef = 0, first_def = 0;                    // parked segments are first_def .. first_def + ndef - 1
     const int vlane = g * G + n;                    // index among the 4G lanes that hold real heads
@@ -265,16 +265,11 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
         for (int k = 0; k < ndef; ++k) {
             const int b = __builtin_amdgcn_readfirstlane(plan[(first_def + k) * kPlanInts]);
             const int64_t slot = (int64_t)h * a.slots_per_head + w + b;
+            // the record leaves as it was parked: all 64 lanes, 16 B each, one contiguous run
             const unsigned char* src = defer + k * slot_bytes;
-            if (n < G) {
-                float* po = a.po + (slot * G + n) * kD + 4 * g;
-#pragma unroll
-                for (int t = 0; t < 8; ++t)
-                    *reinterpret_cast<f32x4*>(po + 16 * t) = *reinterpret_cast<const f32x4*>(src + (vlane * 8 + t) * 16);
-                if (g == 0)
-                    *reinterpret_cast<float2*>(a.ml + (slot * G + n) * 2) =
-                        *reinterpret_cast<const float2*>(src + 512 * G + n * 8);
-            }
+            unsigned char* dst = a.rec + slot * slot_bytes;
+            for (int off = lane * 16; off < slot_bytes; off += 1024)
+                *reinterpret_cast<u32x4*>(dst + off) = *reinterpret_cast<const u32x4*>(src + off);
         }
         first_def += ndef;
         ndef = 0;
@@ -510,8 +505,8 @@ struct MergeArgs {
     int split_workgroups;   // gridDim.x of the split launch that filled the workspace
     const int32_t* seg_first;
     const int32_t* seg_last;
-    const float* ml;
-    const float* po;
+    const unsigned char* rec;
+    int rec_stride;
     int batch;
 };
 
@@ -541,9 +536,10 @@ __global__ void __launch_bounds__(256) paged_decode_merge_kernel(MergeArgs a) {
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int wu = wb + 8 * u <= w1 ? wb + 8 * u : wb;
-            const int64_t row = (slot0 + wu) * G + n;
-            mlv[u] = *reinterpret_cast<const float2*>(a.ml + row * 2);
-            pov[u] = *reinterpret_cast<const f32x4*>(a.po + row * kD + 4 * c4);
+            // columns 4 c4 .. 4 c4 + 3 = accumulator tile t = c4 / 4 of lane group g = c4 % 4
+            const unsigned char* rec = a.rec + (slot0 + wu) * a.rec_stride;
+            mlv[u] = *reinterpret_cast<const float2*>(rec + 512 * G + n * 8);
+            pov[u] = *reinterpret_cast<const f32x4*>(rec + (((c4 & 3) * G + n) * 8 + (c4 >> 2)) * 16);
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -695,8 +691,8 @@ int infer_paged_decode_split_bf16(const void* q, int64_t q_stride0, const void* 
     a.header = (int32_t*)(base + ws.header_off);
     a.seg_first = (int32_t*)(base + ws.seg_first_off);
     a.seg_last = (int32_t*)(base + ws.seg_last_off);
-    a.ml = (float*)(base + ws.ml_off);
-    a.po = (float*)(base + ws.po_off);
+    a.rec = (unsigned char*)base + ws.rec_off;
+    a.rec_stride = (int)ws.rec_stride;
     a.slots_per_head = L.W + (int)batch;
 
     const size_t lds_bytes = (size_t)L.waves * kLdsPerWave;
@@ -736,8 +732,8 @@ int infer_paged_decode_merge_bf16(void* out, int64_t out_stride0, const int32_t*
     m.split_workgroups = L.W;
     m.seg_first = (const int32_t*)(base + ws.seg_first_off);
     m.seg_last = (const int32_t*)(base + ws.seg_last_off);
-    m.ml = (const float*)(base + ws.ml_off);
-    m.po = (const float*)(base + ws.po_off);
+    m.rec = (const unsigned char*)base + ws.rec_off;
+    m.rec_stride = (int)ws.rec_stride;
     m.batch = (int)batch;
     dim3 grid((unsigned)batch, (unsigned)num_q_heads, 1), block(256, 1, 1);
     hipLaunchKernelGGL(paged_decode_merge_kernel, grid, block, 0, (hipStream_t)stream, m);
