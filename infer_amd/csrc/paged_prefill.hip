@@ -242,7 +242,7 @@ constexpr int kQBlock = kNQ * kQTile;
 constexpr int kTileBytes = kStep * kLdsRow;
 
 template <int WAVES>
-__global__ void __launch_bounds__(64 * WAVES) paged_prefill_tile_kernel(PrefillArgs a) {
+__global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) paged_prefill_tile_kernel(PrefillArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_all[];   // [2][K tile | V tile]
     constexpr int kThreads = 64 * WAVES;
     constexpr int kChunks = 512 / kThreads;        // 16-byte chunks of a 32 x 256 B tile per thread
