@@ -237,9 +237,21 @@ __global__ void __launch_bounds__(1024) paged_prefill_kernel(PrefillArgs a) {
 // V tile through LDS.  The tiles are fetched once per workgroup with fully coalesced 16-byte loads,
 // double-buffered (global loads of tile s+1 are in flight while tile s is consumed; one barrier per
 // step), so cache traffic per query drops by 2 G against the one-wave-per-tile kernel above.
+//
+// LDS layout of a tile: key k of the step sits in row  16 ((k >> 2) & 1) + 4 (k >> 3) + (k & 3),  so
+// that the 16 K rows one ds_read_b128 pass touches (one MFMA row tile) and the 8 V rows one
+// transposing read pass touches are consecutive rows.  With a K row stride of 272 B (68 banks:
+// consecutive rows start 4 banks apart) and a V row stride of 288 B (72 banks: 8 apart) both
+// read patterns are free of bank conflicts; the 16-byte stores of a row cover all banks anyway.
 constexpr int kNQ = 2;
+constexpr float kLazy = 8.f;
 constexpr int kQBlock = kNQ * kQTile;
-constexpr int kTileBytes = kStep * kLdsRow;
+constexpr int kKRow = 272;
+constexpr int kVRow = 288;
+constexpr int kKTileBytes = kStep * kKRow;
+constexpr int kVTileBytes = kStep * kVRow;
+constexpr int kTileBytes = kKTileBytes + kVTileBytes;     // one K tile + one V tile
+__device__ __forceinline__ int tile_row(int k) { return 16 * ((k >> 2) & 1) + 4 * (k >> 3) + (k & 3); }
 
 template <int WAVES>
 __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) paged_prefill_tile_kernel(PrefillArgs a) {
@@ -302,42 +314,48 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     // cooperative tile fetch: chunk c covers bytes [16 (c % 16), +16) of row c / 16
     // two tiles are in flight in registers (slots 0 and 1 alternate), a third is being consumed from LDS
     u32x4 kst[2][kChunks], vst[2][kChunks];
+    // chunk i of this thread: row c >> 4 of the tile, 16-byte column c & 15 (both fixed for the kernel)
+    int chunk_row[kChunks], chunk_col[kChunks];
+#pragma unroll
+    for (int i = 0; i < kChunks; ++i) {
+        const int c = tid + i * kThreads;
+        chunk_row[i] = c >> 4;
+        chunk_col[i] = kvh * kD + (c & 15) * 8;
+    }
+    const int tok_stride = (int)a.tok_stride;     // < 2^31 elements (checked on the host)
     auto fetch = [&](auto SLOT, int s) {
         constexpr int S = decltype(SLOT)::value;
         const int tok0 = s * kStep;
-        int64_t base = 0;
+        int64_t base;
         if (a.bt) {
             int blk = __builtin_amdgcn_readfirstlane(a.bt[(int64_t)b * a.bt_stride0 + tok0 / a.block_size]);
             blk = blk < 0 ? 0 : (blk >= a.num_blocks ? a.num_blocks - 1 : blk);
             base = (int64_t)blk * a.blk_stride + (int64_t)(tok0 % a.block_size) * a.tok_stride;
+        } else {
+            base = ((int64_t)k_beg + tok0) * a.tok_stride;
         }
+        // rows past the end of the sequence (last step only) re-read its last row: finite data whose
+        // probabilities are masked to zero, instead of whatever lies behind the sequence
+        const int last = sk - 1 - tok0;
+        const uint16_t* kp = a.k + base;
+        const uint16_t* vp = a.v + base;
 #pragma unroll
         for (int i = 0; i < kChunks; ++i) {
-            const int c = tid + i * kThreads;
-            const int r = c >> 4, col = (c & 15) * 8;
-            int64_t off;
-            if (a.bt) off = base + (int64_t)r * a.tok_stride;
-            else {
-                int64_t row = (int64_t)k_beg + tok0 + r;
-                row = row > a.total_k_rows - 1 ? a.total_k_rows - 1 : row;
-                off = row * a.tok_stride;
-            }
-            off += (int64_t)kvh * kD + col;
-            const bool valid = tok0 + r < sk;      // rows past the sequence may hold anything: read as zeros
-            const u32x4 z = {0u, 0u, 0u, 0u};
-            kst[S][i] = valid ? load16(a.k + off) : z;
-            vst[S][i] = valid ? load16(a.v + off) : z;
+            const int r = chunk_row[i] < last ? chunk_row[i] : last;
+            const int off = r * tok_stride + chunk_col[i];
+            kst[S][i] = load16(kp + off);
+            vst[S][i] = load16(vp + off);
         }
     };
     auto stash = [&](auto SLOT, int buf) {
         constexpr int S = decltype(SLOT)::value;
-        unsigned char* kb = lds_all + buf * 2 * kTileBytes;
+        unsigned char* kb = lds_all + buf * kTileBytes;
 #pragma unroll
         for (int i = 0; i < kChunks; ++i) {
             const int c = tid + i * kThreads;
-            const int off = (c >> 4) * kLdsRow + (c & 15) * 16;
-            *reinterpret_cast<u32x4*>(kb + off) = kst[S][i];
-            *reinterpret_cast<u32x4*>(kb + kTileBytes + off) = vst[S][i];
+            const int row = tile_row(c >> 4);
+            *reinterpret_cast<u32x4*>(kb + row * kKRow + (c & 15) * 16) = kst[S][i];
+            *reinterpret_cast<u32x4*>(kb + kKTileBytes + row * kVRow + (c & 15) * 16) = vst[S][i];
         }
     };
     using S0 = std::integral_constant<int, 0>;
@@ -349,14 +367,13 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     stash(S0{}, 0);
     __syncthreads();
 
-    // K operand row of this lane inside a tile: row r of K tile t holds key 8 (r / 4) + 4 t + r % 4
-    const int krow = 8 * (n >> 2) + (n & 3);
+    // K operand row n of MFMA row tile t is key 8 (n / 4) + 4 t + n % 4, which sits in LDS row 16 t + n
     auto step = [&](auto SLOT, int s) {
         constexpr int S = decltype(SLOT)::value;          // slot of tile s (just consumed from LDS): free again
         using NEXT = std::integral_constant<int, 1 - S>;  // slot of tile s + 1
         if (s + 2 < nsteps) fetch(SLOT, s + 2);
-        const unsigned char* kb = lds_all + (s & 1) * 2 * kTileBytes;
-        const unsigned char* vb = kb + kTileBytes;
+        const unsigned char* kb = lds_all + (s & 1) * kTileBytes;
+        const unsigned char* vb = kb + kKTileBytes;
         const int tok0 = s * kStep;
 
         // ---- S^T = K Q^T for both query tiles
@@ -369,13 +386,16 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const u32x4 kf = *reinterpret_cast<const u32x4*>(kb + (4 * t + krow) * kLdsRow + (32 * j + 8 * g) * 2);
+                const u32x4 kf = *reinterpret_cast<const u32x4*>(kb + (16 * t + n) * kKRow + (32 * j + 8 * g) * 2);
 #pragma unroll
                 for (int u = 0; u < kNQ; ++u)
                     sc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf), qreg[u][j], sc[u][t], 0, 0, 0);
             }
 
-        // ---- online softmax per query tile
+        // ---- online softmax per query tile.  The running maximum is refreshed only when a row's
+        // maximum grows by more than kLazy (log2 units): until then the probabilities are taken
+        // relative to the stale maximum (at most 2^kLazy, harmless in float32 and bf16) and the
+        // accumulators need no rescaling; the final division by the row sum makes both forms equal.
         bf16x8 pb[kNQ];
 #pragma unroll
         for (int u = 0; u < kNQ; ++u) {
@@ -383,7 +403,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) sv[4 * t + e] = sc[u][t][e] * a.scale_log2;
+                for (int e = 0; e < 4; ++e) sv[4 * t + e] = sc[u][t][e];
             if (tok0 + kStep - 1 > my_limit[u]) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i)
@@ -394,30 +414,33 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
             for (int i = 1; i < 8; ++i) mx = fmaxf(mx, sv[i]);
             mx = fmaxf(mx, __shfl_xor(mx, 16));
             mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const float m_new = fmaxf(m_run[u], mx);
-            const float m_ref = m_new == -INFINITY ? 0.f : m_new;
-            const float alpha = __builtin_amdgcn_exp2f(m_run[u] - m_ref);
-            m_run[u] = m_new;
-            float psum = 0.f;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float p = __builtin_amdgcn_exp2f(sv[i] - m_ref);
-                psum += p;
-                pb[u][i] = (__bf16)p;
-            }
-            l_run[u] = l_run[u] * alpha + psum;
-            if (__any(alpha != 1.f)) {
+            mx *= a.scale_log2;                                  // scale > 0: the maximum commutes with it
+            const bool grow = mx > m_run[u] + kLazy;             // -inf + kLazy = -inf: the first finite maximum always grows
+            if (__any(grow)) {
+                const float alpha = grow ? __builtin_amdgcn_exp2f(m_run[u] - mx) : 1.f;
+                m_run[u] = grow ? mx : m_run[u];
+                l_run[u] *= alpha;
 #pragma unroll
                 for (int t = 0; t < 8; ++t) acc[u][t] *= alpha;
             }
+            const float m_neg = m_run[u] == -INFINITY ? 0.f : -m_run[u];
+            float psum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[i], a.scale_log2, m_neg));
+                psum += p;
+                pb[u][i] = (__bf16)p;
+            }
+            l_run[u] += psum;
         }
 
         // ---- O^T += V^T P^T, every V fragment used for both query tiles
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            const unsigned char* src = vb + (8 * g + (n >> 2)) * kLdsRow + (16 * t + 4 * (n & 3)) * 2;
+            // keys 8 g + n / 4 (lo) and 8 g + 4 + n / 4 (hi) sit in LDS rows 4 g + n / 4 and 16 + 4 g + n / 4
+            const unsigned char* src = vb + (4 * g + (n >> 2)) * kVRow + (16 * t + 4 * (n & 3)) * 2;
             const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src));
-            const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src + 4 * kLdsRow));
+            const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src + 16 * kVRow));
             const bf16x8 vt = __builtin_bit_cast(bf16x8, (i16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 #pragma unroll
             for (int u = 0; u < kNQ; ++u)
@@ -457,7 +480,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
 template <int WAVES>
 int launch_tiled(const PrefillArgs& a, int64_t max_seqlen_q, int64_t num_seqs, int64_t num_kv_heads, hipStream_t st) {
     dim3 grid((unsigned)((max_seqlen_q + kQBlock - 1) / kQBlock), (unsigned)num_seqs, (unsigned)num_kv_heads);
-    hipLaunchKernelGGL(paged_prefill_tile_kernel<WAVES>, grid, dim3(64 * WAVES, 1, 1), 4 * kTileBytes, st, a);
+    hipLaunchKernelGGL(paged_prefill_tile_kernel<WAVES>, grid, dim3(64 * WAVES, 1, 1), 2 * kTileBytes, st, a);
     return (int)hipGetLastError();
 }
 
@@ -481,6 +504,7 @@ extern "C" int infer_paged_prefill_bf16(const void* q, int64_t q_stride0, const 
     if (block_table && (kv_block_stride & 7)) return INFER_KV_EALIGN;
     if (kv_token_stride < num_kv_heads * kD || q_stride0 < num_q_heads * kD || out_stride0 < num_q_heads * kD) return INFER_KV_EINVAL;
     if (num_seqs > 65535 || num_kv_heads > 65535) return INFER_KV_EINVAL;
+    if (kv_token_stride > (1 << 24)) return INFER_KV_EUNSUPPORTED;   // 32-bit offsets inside a tile
     const int G = (int)(num_q_heads / num_kv_heads);
     PrefillArgs a;
     a.q = (const uint16_t*)q; a.q_stride0 = q_stride0;
