@@ -113,6 +113,47 @@ def test_graph_replay_is_bit_identical_to_eager_and_padding_rows_touch_nothing(g
     assert (runner.kv_cache[:, :, free] == 77.0).all()       # the padding row wrote to no block
 
 
+def test_graph_replays_at_qwen3_8b_layer_shapes_match_eager(gpu):
+    """Two layers of the real Qwen3-8B geometry (hidden 4096, 32/8 heads, intermediate 12288), batch
+    128: the vendor GEMMs that a replay runs are the ones of the full model.  Five replays, with eager
+    work and synchronisation between them, must each reproduce the eager step bit for bit (a graph
+    node that misbehaves on later replays, such as a memset recorded by a library, would show here)."""
+    from infer_amd.model_runner import ModelRunner
+    from infer_amd.scheduler import Scheduler
+    from infer_amd.sequence import Sequence
+    hf = ModelConfig(vocab_size=2048, hidden_size=4096, intermediate_size=12288, num_hidden_layers=2,
+                     num_attention_heads=32, num_key_value_heads=8, head_dim=128, max_position_embeddings=4096)
+    config = Config(hf_config=hf, num_kvcache_blocks=300, max_model_len=4096, max_num_batched_tokens=16384,
+                    max_num_seqs=128, enforce_eager=False, seed=3)
+    runner = ModelRunner(config)
+    sched = Scheduler(config)
+    g = np.random.default_rng(1)
+    seqs = [Sequence([int(t) for t in g.integers(0, 2048, size=int(n))], SamplingParams(0.0, 8, True))
+            for n in g.integers(64, 300, size=128)]
+    for s in seqs:
+        sched.add(s)
+    while sched.waiting:                                  # the token budget splits the prefill in two
+        batch, is_prefill = sched.schedule()
+        assert is_prefill
+        sched.postprocess(batch, runner.run(batch, True))
+    for step in range(5):
+        batch, is_prefill = sched.schedule()
+        assert not is_prefill and len(batch) == 128
+        run_bs = runner.prepare_decode(batch)
+        assert run_bs == 128
+        with torch.inference_mode():
+            eager = runner._decode_forward(run_bs).clone()
+            reset_context()
+            torch.cuda.synchronize()
+            runner.graphs[run_bs].replay()
+            torch.cuda.synchronize()
+            replay = runner.d_outputs[:run_bs]
+            assert torch.isfinite(replay.float()).all()
+            assert torch.equal(eager, replay), f"replay {step} differs from the eager step"
+            tokens = runner.model.compute_logits(replay).float().argmax(dim=-1).tolist()
+        sched.postprocess(batch, tokens)
+
+
 def test_generate_graph_and_eager_agree_and_prefix_cache_hits(gpu):
     from infer_amd.llm_engine import LLMEngine
     ps = prompts([30, 130, 260, 511], seed=5)
