@@ -122,6 +122,8 @@ def main():
     ap.add_argument("--counters", action="store_true",
                     help="short untimed run for `rocprofv3 --pmc`: a 1 GiB plain copy (x3), the decode op (x5), "
                          "a prefill-sized append (x3)")
+    ap.add_argument("--append-sweep", action="store_true",
+                    help="KV append rate against the number of rows (64 ... 65,536), printed as JSON")
     ap.add_argument("--e2e", action="store_true",
                     help="end-to-end decode through the engine (random-init Qwen3, HIP-graph decode) instead "
                          "of the kernel benchmark")
@@ -175,6 +177,32 @@ def main():
                 ms = gpu_time_ms(cp(wg), 30, 3)
                 res[f"copy_{label}_{wg}wg_GBps_read_plus_write"] = round(2 * nbytes / ms / 1e6, 1)
             del bufs, dst
+        print(json.dumps(res))
+        return
+    if args.append_sweep:
+        # KV append from 64 rows (one decode step) to 65,536 rows: launch-bound at the small end, at the
+        # copy rate of the part at the large end.  Sources and destinations rotate over > 512 MB.
+        dkv, res = 1024, {"append_sweep": True, "row_bytes": 2048, "method": "HIP events, 100 launches after 10 warm-ups"}
+        pool_rows = 1 << 18
+        caches = [(torch.empty((pool_rows // 256, 256, 8, 128), dtype=torch.bfloat16, device=dev),
+                   torch.empty((pool_rows // 256, 256, 8, 128), dtype=torch.bfloat16, device=dev)) for _ in range(2)]
+        for n in (64, 256, 1024, 4096, 16384, 65536):
+            reps = max(2, min(16, (600 << 20) // (n * 4 * dkv)))
+            srcs = [(torch.randn((n, 8, 128), dtype=torch.bfloat16, device=dev),
+                     torch.randn((n, 8, 128), dtype=torch.bfloat16, device=dev)) for _ in range(reps)]
+            slots = [torch.randperm(pool_rows, device=dev)[:n].to(torch.int32) for _ in range(reps)]
+            it = [0]
+
+            def step_append():
+                i = it[0]
+                it[0] += 1
+                kc, vc = caches[i % 2]
+                ops.store_kvcache(srcs[i % reps][0], srcs[i % reps][1], kc, vc, slots[i % reps])
+            ms = gpu_time_ms(step_append, 100, 10)
+            nbytes = workloads.append_algorithmic_bytes(n, n, dkv)
+            res[f"rows_{n}"] = {"us": round(ms * 1e3, 2), "GBps": round(nbytes / ms / 1e6, 1),
+                                "frac_of_8TBps": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+            del srcs, slots
         print(json.dumps(res))
         return
     if args.splits:

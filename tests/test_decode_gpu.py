@@ -42,6 +42,28 @@ def test_cfg1_append_then_decode(gpu):
     print("cfg1 max abs err", err)
 
 
+def test_cfg1_against_the_committed_golden_fixture(gpu):
+    """HIP path against ``tests/golden/cfg1_golden.json``: caches after the append hash to the
+    committed values (bit-exact), the attention output is within the bar of the committed float32
+    output."""
+    import hashlib
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "cfg1_golden.json")) as f:
+        gold = json.load(f)
+    wl = workloads.cfg1().to(gpu)
+    ops.store_kvcache(wl.k_new, wl.v_new, wl.k_cache, wl.v_cache, wl.slot_mapping)
+    torch.cuda.synchronize()
+    sha = lambda t: hashlib.sha256(np.ascontiguousarray(bits(t)).tobytes()).hexdigest()
+    assert sha(wl.k_cache) == gold["after_append_sha256"]["k_cache"]
+    assert sha(wl.v_cache) == gold["after_append_sha256"]["v_cache"]
+    got = f32(gpu_decode(wl))
+    assert list(got.shape) == gold["attention_out"]["shape"]
+    assert np.abs(got[:, :, :8] - np.array(gold["attention_out"]["first8"])).max() <= ATTN_ATOL
+    assert np.abs(got[:, :, -8:] - np.array(gold["attention_out"]["last8"])).max() <= ATTN_ATOL
+    assert np.abs(got.sum(-1) - np.array(gold["attention_out"]["row_sums"])).max() <= 128 * 2 ** -9 * 4
+
+
 @pytest.mark.parametrize("splits", [1, 3, 64, 1024])
 def test_split_count_invariance(gpu, splits):
     wl = workloads.cfg1().to(gpu)

@@ -274,3 +274,19 @@ def test_workload_generator_is_consistent_with_the_metadata_closed_form():
     assert np.array_equal(padded, wl.block_table.numpy())
     flat = [b for t in tables for b in t]
     assert len(set(flat)) == len(flat) == 9      # rows use disjoint blocks: 1 + 1 + 3 + 4
+
+
+def test_cfg1_golden_fixture_is_reproduced_by_generator_and_oracle():
+    """The committed fixture of the reference's CPU-runnable configuration: seeded inputs, caches
+    after the append (bit-exact) and the oracle's attention output must not drift."""
+    import json
+    import os
+    from tests.golden import make_cfg1_golden as G
+    with open(os.path.join(os.path.dirname(G.__file__), "cfg1_golden.json")) as f:
+        want = json.load(f)
+    got = json.loads(json.dumps(G.build()))
+    assert got["config"] == want["config"]
+    assert got["inputs_sha256"] == want["inputs_sha256"]
+    assert got["after_append_sha256"] == want["after_append_sha256"]
+    for key in ("first8", "last8", "row_sums"):
+        assert np.allclose(np.array(got["attention_out"][key]), np.array(want["attention_out"][key]), atol=2e-5)
