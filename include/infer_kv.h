@@ -214,6 +214,18 @@ int infer_decode_metadata(const int32_t* seq_lens, const int32_t* block_table, i
                           int64_t position_offset, int64_t* positions, int32_t* slot_mapping,
                           int32_t* context_lens, void* stream);
 
+/* Replaces Linear.forward (infer/ops/MLP.py:103-149, F.linear; the op matmul(input, weight, output) of
+ * src/bindings.cpp:7) at the batch sizes of a decode step, for weight matrices with few rows (o_proj,
+ * down_proj): y[M, N] = x[M, K] . w[N, K]^T, bf16 in, float32 accumulate, bf16 out, M <= 128.  The
+ * weights (row-major [N, K], contiguous) are streamed from HBM once; K is cut over workgroups and
+ * float32 partial sums pass through `workspace` (infer_skinny_gemm_workspace_bytes says how much,
+ * 0 if the shape needs no split).  K must be a multiple of 128 and N a multiple of 8; other shapes
+ * return INFER_KV_EUNSUPPORTED and belong to the vendor GEMM. */
+size_t infer_skinny_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k);
+int infer_skinny_gemm_bf16(const void* x, int64_t x_stride0, const void* w, void* y, int64_t y_stride0,
+                           int64_t m, int64_t n, int64_t k, void* workspace, size_t workspace_bytes,
+                           void* stream);
+
 /* ------------------------------------------------------------------ measurement helpers
  * No counterpart in the reference.  Plain streaming kernels used by bench.py --ceiling to measure
  * what the part sustains for a read-only stream (same launch shape as the decode kernel: one

@@ -1,7 +1,8 @@
 """The layers of the engine's model around the paged KV-cache path, with the class names and
 forward signatures of the reference (``infer/ops/norm.py``, ``MLP.py``, ``embedding.py``, ``rope.py``,
-``sampler.py``).  GEMMs go to the vendor library through ``F.linear``; normalisation, the SwiGLU gate
-and everything on the cache path are this package's HIP kernels."""
+``sampler.py``).  GEMMs go to the vendor library through ``F.linear``, except decode-sized batches over
+shapes where this package's split-K weight-streaming kernel measures faster (``ops.linear``);
+normalisation, the SwiGLU gate and everything on the cache path are this package's HIP kernels."""
 from __future__ import annotations
 
 import torch
@@ -43,6 +44,8 @@ class Linear(nn.Module):
         param.data.copy_(loaded_weight)
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
+        if self.bias is None and input.dim() == 2 and input.shape[0] <= 128 and input.is_cuda:
+            return ops.linear(input, self.weight)       # decode-sized batch: measured choice of kernel
         return F.linear(input, self.weight, self.bias)
 
 

@@ -279,5 +279,91 @@ def decode_metadata(seq_lens: torch.Tensor, block_table: torch.Tensor, block_siz
     _lib.check(rc, "decode_metadata")
 
 
+_gemm_workspaces: dict = {}
+
+
+def skinny_linear_supported(m: int, n: int, k: int) -> bool:
+    """Shapes the split-K weight-streaming GEMM takes: decode-sized batches over aligned weights."""
+    return 0 < m <= 128 and k % 128 == 0 and n % 8 == 0
+
+
+def skinny_linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``F.linear(x, weight)`` for ``x`` ``[M, K]`` with ``M <= 128`` (``Linear.forward``,
+    ``infer/ops/MLP.py:103-149``): the weight matrix ``[N, K]`` is streamed once by a hand-written
+    split-K kernel.  The float32 workspace is cached per device and only ever grows (a captured graph
+    keeps pointing at the one it was captured with, so outgrown buffers are kept alive)."""
+    m, k = x.shape
+    n = weight.shape[0]
+    assert weight.shape == (n, k) and weight.is_contiguous()
+    assert x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.stride(1) == 1
+    if out is None:
+        out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    assert out.shape == (m, n) and out.dtype == torch.bfloat16 and out.stride(1) == 1
+    _require_gpu(x, weight, out)
+    lib = _lib.load()
+    need = lib.infer_skinny_gemm_workspace_bytes(m, n, k)
+    key = str(x.device)
+    ws = _gemm_workspaces.get(key)
+    if need and (ws is None or ws.numel() < need):
+        if ws is not None:
+            _retired_workspaces.append(ws)
+        ws = torch.empty(max(need, 64 << 20), dtype=torch.uint8, device=x.device)
+        _gemm_workspaces[key] = ws
+    rc = lib.infer_skinny_gemm_bf16(x.data_ptr(), x.stride(0), weight.data_ptr(), out.data_ptr(), out.stride(0),
+                                    m, n, k, ws.data_ptr() if need else None, ws.numel() if need else 0,
+                                    _stream_ptr(x))
+    _lib.check(rc, "skinny_linear")
+    return out
+
+
+_linear_choice: dict = {}
+_flush_buffers: dict = {}
+
+
+def _time_cold(fn, device, reps: int = 6) -> float:
+    """Median GPU time of ``fn`` with the caches flushed before every launch (the weights of a decode
+    step are read once per step, so a warm-cache timing would rank the kernels wrongly)."""
+    flush = _flush_buffers.get(str(device))
+    if flush is None:
+        flush = _flush_buffers[str(device)] = torch.empty(512 << 20, dtype=torch.uint8, device=device)
+    times = []
+    for i in range(reps + 2):
+        flush.zero_()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        fn()
+        end.record()
+        end.synchronize()
+        if i >= 2:
+            times.append(start.elapsed_time(end))
+    times.sort()
+    return times[len(times) // 2]
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """``F.linear(x, weight)`` that sends decode-sized batches to whichever of the vendor GEMM and the
+    split-K weight-streaming kernel is faster for the shape.  The choice is measured once per
+    (device, batch bucket, N, K) with cold caches and kept for the life of the process, so every
+    later call for the shape runs the same kernel; while a HIP graph is being captured nothing is
+    measured (an unknown shape takes the vendor GEMM)."""
+    if x.dim() != 2 or not x.is_cuda or x.dtype != torch.bfloat16:
+        return torch.nn.functional.linear(x, weight)
+    m, k = x.shape
+    n = weight.shape[0]
+    if not skinny_linear_supported(m, n, k) or not weight.is_contiguous() or x.stride(1) != 1:
+        return torch.nn.functional.linear(x, weight)
+    bucket = 16 if m <= 16 else 32 if m <= 32 else 64 if m <= 64 else 128
+    key = (str(x.device), bucket, n, k)
+    use = _linear_choice.get(key)
+    if use is None:
+        if torch.cuda.is_current_stream_capturing():
+            return torch.nn.functional.linear(x, weight)
+        probe = x if m == bucket else torch.zeros((bucket, k), dtype=x.dtype, device=x.device)
+        t_lib = _time_cold(lambda: torch.nn.functional.linear(probe, weight), x.device)
+        t_own = _time_cold(lambda: skinny_linear(probe, weight), x.device)
+        use = _linear_choice[key] = bool(t_own < 0.95 * t_lib)
+    return skinny_linear(x, weight) if use else torch.nn.functional.linear(x, weight)
+
+
 def set_split_workgroups(n: int) -> int:
     return _lib.load().infer_paged_decode_set_split_workgroups(int(n))
