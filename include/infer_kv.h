@@ -225,6 +225,22 @@ size_t infer_skinny_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k);
 int infer_skinny_gemm_bf16(const void* x, int64_t x_stride0, const void* w, void* y, int64_t y_stride0,
                            int64_t m, int64_t n, int64_t k, void* workspace, size_t workspace_bytes,
                            void* stream);
+/* The same product without the final reduction, for a consumer that adds the partial sums itself
+ * (infer_rms_norm_splitk_bf16): *splits_out > 1 means `workspace` now holds float32 partial sums
+ * [splits][m][n] and y was not written; *splits_out == 1 means the shape needed no split and y holds
+ * the bf16 result. */
+int infer_skinny_gemm_partial_bf16(const void* x, int64_t x_stride0, const void* w, void* y, int64_t y_stride0,
+                                   int64_t m, int64_t n, int64_t k, void* workspace, size_t workspace_bytes,
+                                   int* splits_out, void* stream);
+/* infer_rms_norm_bf16 whose input is still in pieces: x[r] = bf16(sum over s of partial[s][r]) with
+ * partial[s][r] at partial + s * split_stride + r * partial_stride0 (float32 elements), added in
+ * split order and rounded once - bit-identical to reducing first - then the same normalisation.
+ * Fuses the reduction of a split-K o_proj / down_proj into the RMSNorm that follows it
+ * (infer/models/Qwen3.py:226-236). */
+int infer_rms_norm_splitk_bf16(const float* partial, int64_t splits, int64_t split_stride,
+                               int64_t partial_stride0, void* residual, int64_t residual_stride0,
+                               const void* weight, void* out, int64_t out_stride0,
+                               int64_t n_rows, int64_t hidden, float eps, void* stream);
 
 /* ------------------------------------------------------------------ measurement helpers
  * No counterpart in the reference.  Plain streaming kernels used by bench.py --ceiling to measure

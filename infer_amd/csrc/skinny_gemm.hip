@@ -222,10 +222,13 @@ extern "C" size_t infer_skinny_gemm_workspace_bytes(int64_t m, int64_t n, int64_
     return s > 1 ? (size_t)s * (size_t)m * (size_t)n * sizeof(float) : 0;
 }
 
-extern "C" int infer_skinny_gemm_bf16(const void* x, int64_t x_stride0, const void* w, void* y, int64_t y_stride0,
-                                      int64_t m, int64_t n, int64_t k, void* workspace, size_t workspace_bytes,
-                                      void* stream) {
+namespace {
+// Launches the streaming kernel and, if asked and the shape was split, the reduction.  Returns the
+// split count through `splits_out`.
+int run_gemm(const void* x, int64_t x_stride0, const void* w, void* y, int64_t y_stride0, int64_t m, int64_t n,
+             int64_t k, void* workspace, size_t workspace_bytes, bool reduce, int* splits_out, void* stream) {
     if (m < 0 || n <= 0 || k <= 0) return INFER_KV_EINVAL;
+    if (splits_out) *splits_out = 0;
     if (m == 0) return INFER_KV_OK;
     if (!x || !w || !y) return INFER_KV_EINVAL;
     if (m > 128 || k % kKC != 0 || n % 8 != 0) return INFER_KV_EUNSUPPORTED;
@@ -245,9 +248,24 @@ extern "C" int infer_skinny_gemm_bf16(const void* x, int64_t x_stride0, const vo
     else if (m <= 64) hipLaunchKernelGGL(skinny_gemm_kernel<4>, grid, dim3(256), 0, st, a);
     else hipLaunchKernelGGL(skinny_gemm_kernel<8>, grid, dim3(256), 0, st, a);
     int rc = (int)hipGetLastError();
-    if (rc != 0 || splits == 1) return rc;
+    if (splits_out) *splits_out = splits;
+    if (rc != 0 || splits == 1 || !reduce) return rc;
     ReduceArgs r{(const float*)workspace, (uint16_t*)y, y_stride0, (int)m, (int)n, splits};
     const int64_t items = m * (n / 8);
     hipLaunchKernelGGL(skinny_gemm_reduce_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, r);
     return (int)hipGetLastError();
+}
+}  // namespace
+
+extern "C" int infer_skinny_gemm_bf16(const void* x, int64_t x_stride0, const void* w, void* y, int64_t y_stride0,
+                                      int64_t m, int64_t n, int64_t k, void* workspace, size_t workspace_bytes,
+                                      void* stream) {
+    return run_gemm(x, x_stride0, w, y, y_stride0, m, n, k, workspace, workspace_bytes, true, nullptr, stream);
+}
+
+extern "C" int infer_skinny_gemm_partial_bf16(const void* x, int64_t x_stride0, const void* w, void* y,
+                                              int64_t y_stride0, int64_t m, int64_t n, int64_t k, void* workspace,
+                                              size_t workspace_bytes, int* splits_out, void* stream) {
+    if (!splits_out) return INFER_KV_EINVAL;
+    return run_gemm(x, x_stride0, w, y, y_stride0, m, n, k, workspace, workspace_bytes, false, splits_out, stream);
 }

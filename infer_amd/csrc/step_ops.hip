@@ -17,6 +17,7 @@
 namespace {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
@@ -36,10 +37,12 @@ __device__ __forceinline__ u32x4 pack8(const float (&x)[8]) {
     return r;
 }
 
-constexpr int kNormThreads = 256;
-constexpr int kNormMaxChunks = 4;   // 16-byte chunks per thread: hidden <= 256 * 4 * 8 = 8192
+constexpr int kNormThreads = 512;
+constexpr int kNormMaxChunks = 2;   // 16-byte chunks per thread: hidden <= 512 * 2 * 8 = 8192
 
 struct NormArgs {
+    const float* partial;      // if set: x[row] = bf16(sum over splits of partial[s][row]) instead of reading x
+    int splits; int64_t split_stride; int64_t partial_stride0;
     const uint16_t* x; int64_t x_stride0;
     uint16_t* residual; int64_t residual_stride0;
     const uint16_t* weight;
@@ -49,7 +52,7 @@ struct NormArgs {
     float eps;
 };
 
-// One workgroup per row.  The row (plus residual) is held in registers as float32 between the two
+// One workgroup of 512 threads per row (one or two 16-byte chunks per thread: many loads in flight).  The row (plus residual) is held in registers as float32 between the two
 // passes, so each input byte is read once.  Rounding points of the reference: the residual output
 // is bf16(x + residual) while the variance and the scaling use the unrounded float32 sum; the
 // scaled value is rounded to bf16 and then multiplied by the bf16 weight (rounded again).
@@ -65,7 +68,20 @@ __global__ void __launch_bounds__(kNormThreads) rms_norm_kernel(NormArgs a) {
     for (int j = 0; j < kNormMaxChunks; ++j) {
         const int c = tid + j * kNormThreads;
         if (c < a.chunks) {
-            unpack8(*reinterpret_cast<const u32x4*>(xr + 8 * c), v[j]);
+            if (a.partial) {
+                // split-K partial sums of the producing GEMM, added in split order and rounded to bf16
+                // once, exactly as the GEMM's own reduction kernel would have done
+                const float* pp = a.partial + row * a.partial_stride0 + 8 * c;
+                f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
+                for (int s = 0; s < a.splits; ++s) {
+                    lo += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(pp + s * a.split_stride));
+                    hi += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(pp + s * a.split_stride + 4));
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { v[j][e] = rb(lo[e]); v[j][4 + e] = rb(hi[e]); }
+            } else {
+                unpack8(*reinterpret_cast<const u32x4*>(xr + 8 * c), v[j]);
+            }
             if (rr) {
                 float r[8];
                 unpack8(*reinterpret_cast<const u32x4*>(rr + 8 * c), r);
@@ -82,7 +98,9 @@ __global__ void __launch_bounds__(kNormThreads) rms_norm_kernel(NormArgs a) {
     __shared__ float part[kNormThreads / 64];
     if ((tid & 63) == 0) part[tid >> 6] = ss;
     __syncthreads();
-    ss = part[0] + part[1] + part[2] + part[3];
+    ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < kNormThreads / 64; ++i) ss += part[i];
     const float rs = rsqrtf(ss * a.inv_hidden + a.eps);
 
     uint16_t* orow = a.out + row * a.out_stride0;
@@ -168,8 +186,28 @@ extern "C" int infer_rms_norm_bf16(const void* x, int64_t x_stride0, void* resid
     if (!aligned16(x) || !aligned16(weight) || !aligned16(out) || !aligned16(residual) || x_stride0 % 8 ||
         out_stride0 % 8 || (residual && residual_stride0 % 8))
         return INFER_KV_EALIGN;
-    NormArgs a{(const uint16_t*)x, x_stride0, (uint16_t*)residual, residual_stride0, (const uint16_t*)weight,
-               (uint16_t*)out, out_stride0, (int)(hidden / 8), 1.0f / (float)hidden, eps};
+    NormArgs a{nullptr, 0, 0, 0, (const uint16_t*)x, x_stride0, (uint16_t*)residual, residual_stride0,
+               (const uint16_t*)weight, (uint16_t*)out, out_stride0, (int)(hidden / 8), 1.0f / (float)hidden, eps};
+    hipLaunchKernelGGL(rms_norm_kernel, dim3((unsigned)n_rows), dim3(kNormThreads), 0, (hipStream_t)stream, a);
+    return (int)hipGetLastError();
+}
+
+extern "C" int infer_rms_norm_splitk_bf16(const float* partial, int64_t splits, int64_t split_stride,
+                                          int64_t partial_stride0, void* residual, int64_t residual_stride0,
+                                          const void* weight, void* out, int64_t out_stride0, int64_t n_rows,
+                                          int64_t hidden, float eps, void* stream) {
+    if (n_rows < 0 || hidden <= 0 || splits <= 0 || splits > 64) return INFER_KV_EINVAL;
+    if (n_rows == 0) return INFER_KV_OK;
+    if (!partial || !weight || !out) return INFER_KV_EINVAL;
+    if (hidden % 8 != 0 || hidden > 8 * kNormThreads * kNormMaxChunks) return INFER_KV_EUNSUPPORTED;
+    if (n_rows > 0x7fffffff) return INFER_KV_EINVAL;
+    if (partial_stride0 < hidden || out_stride0 < hidden || (residual && residual_stride0 < hidden)) return INFER_KV_EINVAL;
+    if (splits > 1 && split_stride < n_rows * partial_stride0) return INFER_KV_EINVAL;
+    if (!aligned16(partial) || !aligned16(weight) || !aligned16(out) || !aligned16(residual) || partial_stride0 % 4 ||
+        split_stride % 4 || out_stride0 % 8 || (residual && residual_stride0 % 8))
+        return INFER_KV_EALIGN;
+    NormArgs a{partial, (int)splits, split_stride, partial_stride0, nullptr, 0, (uint16_t*)residual, residual_stride0,
+               (const uint16_t*)weight, (uint16_t*)out, out_stride0, (int)(hidden / 8), 1.0f / (float)hidden, eps};
     hipLaunchKernelGGL(rms_norm_kernel, dim3((unsigned)n_rows), dim3(kNormThreads), 0, (hipStream_t)stream, a);
     return (int)hipGetLastError();
 }

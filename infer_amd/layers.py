@@ -43,9 +43,11 @@ class Linear(nn.Module):
     def weight_loader(param: nn.Parameter, loaded_weight: torch.Tensor):
         param.data.copy_(loaded_weight)
 
-    def forward(self, input: torch.Tensor) -> torch.Tensor:
+    def forward(self, input: torch.Tensor, defer: bool = False):
+        """``defer=True`` is for a caller that passes the result straight to an ``RMSNorm``: a split-K
+        result may then come back unreduced (``ops.SplitKSum``) and the norm kernel adds the pieces."""
         if self.bias is None and input.dim() == 2 and input.shape[0] <= 128 and input.is_cuda:
-            return ops.linear(input, self.weight)       # decode-sized batch: measured choice of kernel
+            return ops.linear(input, self.weight, defer)    # decode-sized batch: measured choice of kernel
         return F.linear(input, self.weight, self.bias)
 
 
@@ -90,7 +92,7 @@ class MLP(nn.Module):
         x = self.gate_up_proj(x)
         act = torch.empty(x.shape[:-1] + (self.intermediate_size,), dtype=x.dtype, device=x.device)
         ops.silu_and_mul(act, x)
-        return self.down_proj(act)
+        return self.down_proj(act, defer=True)      # consumed by the next RMSNorm (with its residual add)
 
 
 class Embedding(nn.Module):

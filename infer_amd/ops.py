@@ -11,6 +11,8 @@ current stream.  Tensors must live on the GPU; there is no CPU path.
 """
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 from . import _lib
@@ -225,6 +227,8 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.
              out: torch.Tensor | None = None):
     """``RMSNorm.forward`` of ``infer/ops/norm.py:63-98``: returns ``out`` or, with ``residual``,
     ``(out, residual)`` where ``residual`` has been updated in place to ``x + residual``."""
+    if isinstance(x, SplitKSum):
+        return _rms_norm_splitk(x, weight, eps, residual, out)
     hidden = x.shape[-1]
     x2 = x.reshape(-1, hidden)
     assert x2.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x2.stride(1) == 1
@@ -243,6 +247,29 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.
         r2.stride(0) if r2 is not None else 0, weight.data_ptr(), o2.data_ptr(), o2.stride(0),
         x2.shape[0], hidden, float(eps), _stream_ptr(x))
     _lib.check(rc, "rms_norm")
+    return out if residual is None else (out, residual)
+
+
+def _rms_norm_splitk(x: "SplitKSum", weight, eps, residual, out):
+    """RMSNorm over a split-K GEMM result that is still in pieces: the kernel adds the partial sums
+    (in split order, rounded to bf16 once: the same bits as reducing first) and normalises."""
+    x.check_alive()
+    p = x.partial
+    splits, m, hidden = p.shape
+    assert p.dtype == torch.float32 and p.is_contiguous()
+    assert weight.dtype == torch.bfloat16 and weight.shape == (hidden,) and weight.is_contiguous()
+    if out is None:
+        out = torch.empty((m, hidden), dtype=x.dtype, device=p.device)
+    assert out.shape == (m, hidden) and out.dtype == torch.bfloat16 and out.stride(1) == 1
+    r2 = None
+    if residual is not None:
+        r2 = residual.view(-1, hidden)
+        assert r2.shape == (m, hidden) and r2.dtype == torch.bfloat16 and r2.stride(1) == 1
+    rc = _lib.load().infer_rms_norm_splitk_bf16(
+        p.data_ptr(), splits, m * hidden, hidden, r2.data_ptr() if r2 is not None else None,
+        r2.stride(0) if r2 is not None else 0, weight.data_ptr(), out.data_ptr(), out.stride(0), m, hidden,
+        float(eps), _stream_ptr(p))
+    _lib.check(rc, "rms_norm (split-K input)")
     return out if residual is None else (out, residual)
 
 
@@ -287,6 +314,70 @@ def skinny_linear_supported(m: int, n: int, k: int) -> bool:
     return 0 < m <= 128 and k % 128 == 0 and n % 8 == 0
 
 
+def _gemm_workspace(device, need: int) -> torch.Tensor | None:
+    key = str(device)
+    ws = _gemm_workspaces.get(key)
+    if need and (ws is None or ws.numel() < need):
+        if ws is not None:
+            _retired_workspaces.append(ws)
+        ws = torch.empty(max(need, 64 << 20), dtype=torch.uint8, device=device)
+        _gemm_workspaces[key] = ws
+    return ws
+
+
+class SplitKSum:
+    """Result of a split-K GEMM that has not been reduced yet: ``partial`` ``[splits, M, N]`` float32
+    lives in the shared GEMM workspace, so it must be consumed (``rms_norm`` does, ``materialize``
+    does) before the next split-K GEMM on the device runs; ``generation`` guards that."""
+    _generation: dict = {}
+
+    def __init__(self, partial: torch.Tensor, dtype):
+        self.partial = partial
+        self.dtype = dtype
+        key = str(partial.device)
+        self.generation = SplitKSum._generation[key] = SplitKSum._generation.get(key, 0) + 1
+
+    @property
+    def shape(self):
+        return self.partial.shape[1:]
+
+    def check_alive(self):
+        if SplitKSum._generation.get(str(self.partial.device)) != self.generation:
+            raise RuntimeError("split-K partial sums were overwritten by a later GEMM before they were consumed")
+
+    def materialize(self) -> torch.Tensor:
+        self.check_alive()
+        total = self.partial[0].clone()
+        for s in range(1, self.partial.shape[0]):      # split order, as the kernels add them
+            total += self.partial[s]
+        return total.to(self.dtype)
+
+
+def skinny_linear_deferred(x: torch.Tensor, weight: torch.Tensor):
+    """``skinny_linear`` that leaves the split-K reduction to its consumer: returns a ``SplitKSum`` when
+    the shape was split, the finished bf16 tensor otherwise."""
+    m, k = x.shape
+    n = weight.shape[0]
+    assert weight.shape == (n, k) and weight.is_contiguous()
+    assert x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.stride(1) == 1
+    _require_gpu(x, weight)
+    lib = _lib.load()
+    need = lib.infer_skinny_gemm_workspace_bytes(m, n, k)
+    out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    if not need:
+        return skinny_linear(x, weight, out)
+    ws = _gemm_workspace(x.device, need)
+    splits = ctypes.c_int(0)
+    rc = lib.infer_skinny_gemm_partial_bf16(x.data_ptr(), x.stride(0), weight.data_ptr(), out.data_ptr(),
+                                            out.stride(0), m, n, k, ws.data_ptr(), ws.numel(),
+                                            ctypes.byref(splits), _stream_ptr(x))
+    _lib.check(rc, "skinny_linear_deferred")
+    if splits.value <= 1:
+        return out
+    partial = ws[:splits.value * m * n * 4].view(torch.float32).view(splits.value, m, n)
+    return SplitKSum(partial, x.dtype)
+
+
 def skinny_linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
     """``F.linear(x, weight)`` for ``x`` ``[M, K]`` with ``M <= 128`` (``Linear.forward``,
     ``infer/ops/MLP.py:103-149``): the weight matrix ``[N, K]`` is streamed once by a hand-written
@@ -302,13 +393,9 @@ def skinny_linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | Non
     _require_gpu(x, weight, out)
     lib = _lib.load()
     need = lib.infer_skinny_gemm_workspace_bytes(m, n, k)
-    key = str(x.device)
-    ws = _gemm_workspaces.get(key)
-    if need and (ws is None or ws.numel() < need):
-        if ws is not None:
-            _retired_workspaces.append(ws)
-        ws = torch.empty(max(need, 64 << 20), dtype=torch.uint8, device=x.device)
-        _gemm_workspaces[key] = ws
+    ws = _gemm_workspace(x.device, need)
+    if need:      # any unconsumed SplitKSum in this workspace is gone after this launch
+        SplitKSum._generation[str(x.device)] = SplitKSum._generation.get(str(x.device), 0) + 1
     rc = lib.infer_skinny_gemm_bf16(x.data_ptr(), x.stride(0), weight.data_ptr(), out.data_ptr(), out.stride(0),
                                     m, n, k, ws.data_ptr() if need else None, ws.numel() if need else 0,
                                     _stream_ptr(x))
@@ -340,7 +427,7 @@ def _time_cold(fn, device, reps: int = 6) -> float:
     return times[len(times) // 2]
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+def linear(x: torch.Tensor, weight: torch.Tensor, defer: bool = False):
     """``F.linear(x, weight)`` that sends decode-sized batches to whichever of the vendor GEMM and the
     split-K weight-streaming kernel is faster for the shape.  The choice is measured once per
     (device, batch bucket, N, K) with cold caches and kept for the life of the process, so every
@@ -362,7 +449,10 @@ def linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
         t_lib = _time_cold(lambda: torch.nn.functional.linear(probe, weight), x.device)
         t_own = _time_cold(lambda: skinny_linear(probe, weight), x.device)
         use = _linear_choice[key] = bool(t_own < 0.95 * t_lib)
-    return skinny_linear(x, weight) if use else torch.nn.functional.linear(x, weight)
+    if not use:
+        return torch.nn.functional.linear(x, weight)
+    # ``defer``: the caller hands the result straight to ``rms_norm``, which adds the partial sums itself
+    return skinny_linear_deferred(x, weight) if defer else skinny_linear(x, weight)
 
 
 def set_split_workgroups(n: int) -> int:

@@ -63,7 +63,7 @@ class QwenAttention(nn.Module):
         ops.qk_norm_rope_store_kvcache(q, k, v, positions, self.q_norm.weight, self.k_norm.weight,
                                        self.q_norm.eps, table, k_cache, v_cache, slots, write_key=keys_from_rows)
         o = self.attn(q, k, v, kv_stored=True)
-        return self.o_proj(o)
+        return self.o_proj(o, defer=True)           # consumed by post_attention_layernorm
 
 
 class QwenDecoderLayer(nn.Module):

@@ -84,3 +84,35 @@ def test_linear_picks_one_kernel_per_shape_and_matches(gpu):
     close(a, reference(x, w))
     big = torch.randn(300, 12288, generator=g).to(torch.bfloat16).to(gpu)
     close(ops.linear(big, w), reference(big, w))         # larger batches take the vendor GEMM
+
+
+@pytest.mark.parametrize("m,n,k,with_residual", [(128, 4096, 12288, True), (40, 4096, 4096, True), (7, 1024, 2048, False)])
+def test_rms_norm_adds_unreduced_partial_sums_to_the_same_bits(gpu, m, n, k, with_residual):
+    """RMSNorm fed with the unreduced split-K result must give exactly what reducing first gives."""
+    g = torch.Generator().manual_seed(m + k)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16).to(gpu)
+    w = (torch.randn(n, k, generator=g) * 0.03).to(torch.bfloat16).to(gpu)
+    gamma = (1 + 0.2 * torch.randn(n, generator=g)).to(torch.bfloat16).to(gpu)
+    res_a = torch.randn(m, n, generator=g).to(torch.bfloat16).to(gpu) if with_residual else None
+    res_b = res_a.clone() if with_residual else None
+    finished = ops.skinny_linear(x, w)
+    want = ops.rms_norm(finished, gamma, 1e-6, res_a)
+    deferred = ops.skinny_linear_deferred(x, w)
+    assert isinstance(deferred, ops.SplitKSum) and deferred.partial.shape[0] > 1
+    assert torch.equal(deferred.materialize(), finished)
+    got = ops.rms_norm(deferred, gamma, 1e-6, res_b)
+    torch.cuda.synchronize()
+    if with_residual:
+        assert torch.equal(got[0], want[0]) and torch.equal(res_b, res_a)
+    else:
+        assert torch.equal(got, want)
+
+
+def test_partial_sums_cannot_be_used_after_a_later_split_gemm(gpu):
+    x = torch.zeros(8, 4096, dtype=torch.bfloat16, device=gpu)
+    w = torch.zeros(1024, 4096, dtype=torch.bfloat16, device=gpu)
+    first = ops.skinny_linear_deferred(x, w)
+    assert isinstance(first, ops.SplitKSum)
+    ops.skinny_linear_deferred(x, w)
+    with pytest.raises(RuntimeError, match="overwritten"):
+        ops.rms_norm(first, torch.ones(1024, dtype=torch.bfloat16, device=gpu), 1e-6)
