@@ -14,12 +14,11 @@ What differs from the reference, by design for this hardware:
 """
 from __future__ import annotations
 
-import numpy as np
 import torch
 
 from . import kv_runner, ops
 from .config import Config
-from .context import get_context, reset_context, set_context
+from .context import reset_context, set_context
 from .layers import Sampler
 from .qwen3 import QwenForCausalLM, init_random_weights
 from .sampling_params import SamplingParams

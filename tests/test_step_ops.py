@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from oracle import step_ops_ref as S
-from oracle.paged_ref import bf16_to_f32, decode_metadata_ref, f32_to_bf16
+from oracle.paged_ref import bf16_to_f32, decode_metadata_ref
 from tests.helpers import bits
 
 
