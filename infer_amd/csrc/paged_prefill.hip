@@ -6,14 +6,18 @@
 // of its paged cache; without one K and V are the packed new rows.  The causal mask is aligned to
 // the bottom-right corner: key j is visible to query i iff j <= i + (sk - sq).
 //
-// One wavefront owns 16 consecutive queries of one query head and walks the visible keys in steps
-// of 32, with the same arithmetic as the decode kernel, the 16 MFMA columns now being 16 queries
-// instead of the heads of a GQA group:
-//   S^T[key, query] = K[key, :] . Q^T       2 tiles x 4 v_mfma_f32_16x16x32_bf16
+// A wavefront owns 32 consecutive queries (two MFMA column tiles) of one query head and walks the
+// visible keys in steps of 32, with the arithmetic of the decode kernel, the MFMA columns now being
+// queries instead of the heads of a GQA group:
+//   S^T[key, query] = K[key, :] . Q^T       2 row tiles x 4 v_mfma_f32_16x16x32_bf16 per column tile
 //   online softmax in the accumulator layout (lane = query, 8 keys per lane)
-//   O^T[d, query]  += V^T[d, key] . P^T     8 MFMAs, V staged through a wave-private LDS tile
-// The G wavefronts of a workgroup are the G query heads that share one KV head and the same query
-// tile, so they read the same K/V rows at about the same time (cache hits).
+//   O^T[d, query]  += V^T[d, key] . P^T     8 MFMAs per column tile
+// A workgroup is 4 to 8 wavefronts that read the same keys: the query heads of one KV head (all of
+// them, or a divisor-sized part when the group is larger than 8) times as many consecutive query
+// blocks as fit (4 blocks for a group of 1, 2 for groups of 2 and 3, 1 otherwise).  They share
+// every 32-key K tile and V tile through LDS: the tiles are fetched once per workgroup with fully
+// coalesced 16-byte loads and double-buffered (the loads of tile s + 2 are in flight in registers
+// while tile s + 1 sits in LDS and tile s is consumed; one barrier per step).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -34,9 +38,6 @@ typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
 constexpr int kD = 128;
 constexpr int kStep = 32;        // keys per step
 constexpr int kQTile = 16;       // queries per wavefront
-constexpr int kLdsRow = 288;     // 256 + 32: four consecutive rows hit disjoint LDS banks
-constexpr int kLdsWave = kStep * kLdsRow;
-
 struct PrefillArgs {
     const uint16_t* q;
     int64_t q_stride0;
@@ -50,10 +51,11 @@ struct PrefillArgs {
     const int32_t* cu_k;
     const int32_t* bt;      // nullptr: packed K/V
     int64_t bt_stride0;
-    int group;
+    int group;              // query heads per KV head
+    int heads_per_wg;       // query heads of the group that one workgroup covers (divides group)
+    int qblocks_per_wg;     // consecutive query blocks one workgroup covers
     int block_size;
     int num_blocks;
-    int64_t total_k_rows;   // packed mode: rows in k/v (for clamping the tail)
     float scale_log2;
     int causal;
 };
@@ -62,182 +64,6 @@ __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 x) { return __builtin_bit_cast
 __device__ __forceinline__ u32x4 load16(const uint16_t* p) { return *reinterpret_cast<const u32x4*>(p); }
 __device__ __forceinline__ void lds_order() { __asm__ volatile("" ::: "memory"); }
 
-__global__ void __launch_bounds__(1024) paged_prefill_kernel(PrefillArgs a) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds_all[];
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int g = lane >> 4, n = lane & 15;
-    const int b = blockIdx.y;
-    const int kvh = blockIdx.z;
-    const int head = kvh * a.group + wave;
-    unsigned char* lds = lds_all + wave * kLdsWave;
-
-    const int q_beg = a.cu_q[b], q_end = a.cu_q[b + 1];
-    const int k_beg = a.cu_k[b], k_end = a.cu_k[b + 1];
-    const int sq = q_end - q_beg, sk = k_end - k_beg;
-    const int q0 = blockIdx.x * kQTile;
-    if (q0 >= sq || sk <= 0) {
-        // queries without any key produce zeros (only possible when sk == 0)
-        if (q0 + n < sq && sk <= 0) {
-            uint16_t* op = a.out + (int64_t)(q_beg + q0 + n) * a.out_stride0 + (int64_t)head * kD + 4 * g;
-            for (int t = 0; t < 8; ++t) *reinterpret_cast<u32x2*>(op + 16 * t) = u32x2{0u, 0u};
-        }
-        return;
-    }
-    const int shift = sk - sq;                       // bottom-right alignment
-    const int my_q = q0 + n;                         // this lane's query (may be past sq: padded column)
-    const int my_limit = a.causal ? (my_q + shift < sk - 1 ? my_q + shift : sk - 1) : sk - 1;   // last visible key
-    int tile_last = q0 + kQTile - 1 < sq - 1 ? q0 + kQTile - 1 : sq - 1;
-    const int key_end = a.causal ? (tile_last + shift + 1 < sk ? tile_last + shift + 1 : sk) : sk;   // keys [0, key_end)
-    const int nsteps = (key_end + kStep - 1) / kStep;
-
-    // Q as the B operand: lane (g, n) holds Q[query n][32 j + 8 g .. +8]
-    bf16x8 qreg[4];
-    {
-        const u32x4 z = {0u, 0u, 0u, 0u};
-        const bool live = my_q < sq;
-        const uint16_t* qp = a.q + (int64_t)(q_beg + (live ? my_q : 0)) * a.q_stride0 + (int64_t)head * kD + 8 * g;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) qreg[j] = as_bf16x8(live ? load16(qp + 32 * j) : z);
-    }
-
-    f32x4 acc[8];
-#pragma unroll
-    for (int t = 0; t < 8; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float m_run = -INFINITY, l_run = 0.f;
-
-    // row r of K tile t holds key 8 (r / 4) + 4 t + r % 4 of the step: lane group g ends up with keys 8 g .. 8 g + 7
-    const int krow = 8 * (n >> 2) + (n & 3);
-    u32x4 kreg[2][4];
-    u32x4 vreg[8];
-
-    auto issue_loads = [&](int s) {
-        const int tok0 = s * kStep;
-        if (a.bt) {
-            int blk = __builtin_amdgcn_readfirstlane(a.bt[(int64_t)b * a.bt_stride0 + tok0 / a.block_size]);
-            blk = blk < 0 ? 0 : (blk >= a.num_blocks ? a.num_blocks - 1 : blk);
-            const int64_t base = (int64_t)blk * a.blk_stride + (int64_t)(tok0 % a.block_size) * a.tok_stride + (int64_t)kvh * kD;
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    kreg[t][j] = load16(a.k + base + (int64_t)(4 * t + krow) * a.tok_stride + 8 * g + 32 * j);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) vreg[i] = load16(a.v + base + (int64_t)(4 * i + g) * a.tok_stride + 8 * n);
-        } else {
-            const int64_t row0 = (int64_t)k_beg + tok0;
-            const int64_t last = a.total_k_rows - 1;
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                int64_t r = row0 + 4 * t + krow;
-                r = r > last ? last : r;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) kreg[t][j] = load16(a.k + r * a.tok_stride + (int64_t)kvh * kD + 8 * g + 32 * j);
-            }
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                int64_t r = row0 + 4 * i + g;
-                r = r > last ? last : r;
-                vreg[i] = load16(a.v + r * a.tok_stride + (int64_t)kvh * kD + 8 * n);
-            }
-        }
-    };
-
-    issue_loads(0);
-    for (int s = 0; s < nsteps; ++s) {
-        f32x4 sc[2];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            sc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kreg[t][j]), qreg[j], sc[t], 0, 0, 0);
-        }
-        const int tok0 = s * kStep;
-        // rows past the end of the sequence may hold anything: zero them in V (0 * NaN must not leak)
-        if (tok0 + kStep > sk) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                if (tok0 + 4 * i + g >= sk) vreg[i] = u32x4{0u, 0u, 0u, 0u};
-        }
-        lds_order();
-#pragma unroll
-        for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(lds + (4 * i + g) * kLdsRow + n * 16) = vreg[i];
-        lds_order();
-        if (s + 1 < nsteps) issue_loads(s + 1);
-
-        float sv[8];
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) sv[4 * t + e] = sc[t][e] * a.scale_log2;
-        if (tok0 + kStep - 1 > my_limit) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                if (tok0 + 8 * g + i > my_limit) sv[i] = -INFINITY;
-        }
-        float mx = sv[0];
-#pragma unroll
-        for (int i = 1; i < 8; ++i) mx = fmaxf(mx, sv[i]);
-        mx = fmaxf(mx, __shfl_xor(mx, 16));
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx);
-        // a query that has seen no key yet keeps m = -inf: use 0 as the reference point then
-        const float m_ref = m_new == -INFINITY ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
-        m_run = m_new;
-        float psum = 0.f;
-        float pv[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            pv[i] = __builtin_amdgcn_exp2f(sv[i] - m_ref);
-            psum += pv[i];
-        }
-        l_run = l_run * alpha + psum;
-        bf16x8 pb;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) pb[i] = (__bf16)pv[i];
-        if (__any(alpha != 1.f)) {
-#pragma unroll
-            for (int t = 0; t < 8; ++t) acc[t] *= alpha;
-        }
-        // A operand element i of lane (g, n) is V[key 8 g + i][16 t + n], fetched with the transposing
-        // LDS read: in each group of 16 lanes, lane i points at row i / 4, column quad i % 4, and lane l
-        // receives column l of those four rows.
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            const unsigned char* src = lds + (8 * g + (n >> 2)) * kLdsRow + (16 * t + 4 * (n & 3)) * 2;
-            const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src));
-            const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src + 4 * kLdsRow));
-            const i16x8 vt = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vt), pb, acc[t], 0, 0, 0);
-        }
-        lds_order();
-    }
-
-    l_run += __shfl_xor(l_run, 16);
-    l_run += __shfl_xor(l_run, 32);
-    if (my_q < sq) {
-        const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
-        uint16_t* op = a.out + (int64_t)(q_beg + my_q) * a.out_stride0 + (int64_t)head * kD + 4 * g;
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            union { __bf16 hv[4]; u32x2 u; } r;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) r.hv[e] = (__bf16)(acc[t][e] * inv);
-            *reinterpret_cast<u32x2*>(op + 16 * t) = r.u;
-        }
-    }
-}
-
-
-// ---------------------------------------------------------------------------------------------
-// Tiled variant, used when the GQA group size is 1, 2, 4 or 8: the WAVES = G wavefronts of a
-// workgroup (one query head each, 32 queries = 2 MFMA column tiles) share every 32-key K tile and
-// V tile through LDS.  The tiles are fetched once per workgroup with fully coalesced 16-byte loads,
-// double-buffered (global loads of tile s+1 are in flight while tile s is consumed; one barrier per
-// step), so cache traffic per query drops by 2 G against the one-wave-per-tile kernel above.
-//
 // LDS layout of a tile: key k of the step sits in row  16 ((k >> 2) & 1) + 4 (k >> 3) + (k & 3),  so
 // that the 16 K rows one ds_read_b128 pass touches (one MFMA row tile) and the 8 V rows one
 // transposing read pass touches are consecutive rows.  With a row stride of 272 B (68 banks:
@@ -253,29 +79,38 @@ constexpr int kVTileBytes = kStep * kVRow;
 constexpr int kTileBytes = kKTileBytes + kVTileBytes;     // one K tile + one V tile
 __device__ __forceinline__ int tile_row(int k) { return 16 * ((k >> 2) & 1) + 4 * (k >> 3) + (k & 3); }
 
-template <int WAVES>
+// WAVES = heads per workgroup x QB, QB = query blocks per workgroup (a compile-time constant so that the
+// common QB == 1 case carries no per-wavefront step guard).
+template <int WAVES, int QB>
 __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) paged_prefill_tile_kernel(PrefillArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_all[];   // [2][K tile | V tile]
     constexpr int kThreads = 64 * WAVES;
-    constexpr int kChunks = 512 / kThreads;        // 16-byte chunks of a 32 x 256 B tile per thread
+    constexpr int kTileChunks = kStep * 16;                            // 16-byte chunks of a 32 x 256 B tile
+    constexpr int kChunks = (kTileChunks + kThreads - 1) / kThreads;   // tile chunks per thread
+    constexpr bool kRagged = kTileChunks % kThreads != 0;              // the last round is only partly used
+    constexpr int kHeads = WAVES / QB;                                 // query heads per workgroup
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane >> 4, n = lane & 15;
     const int b = blockIdx.y;
-    const int kvh = blockIdx.z;
-    const int head = kvh * WAVES + wave;
+    const int parts = a.group / kHeads;                    // workgroups that share one KV head
+    const int kvh = blockIdx.z / parts;
+    const int head = kvh * a.group + (blockIdx.z % parts) * kHeads + (QB == 1 ? wave : wave % kHeads);
+    const int qb = QB == 1 ? 0 : wave / kHeads;            // query block of this wavefront inside the workgroup
 
     const int q_beg = a.cu_q[b], q_end = a.cu_q[b + 1];
     const int k_beg = a.cu_k[b], k_end = a.cu_k[b + 1];
     const int sq = q_end - q_beg, sk = k_end - k_beg;
     // late query blocks see the most keys: hand them out first so the long workgroups start early
-    const int q0 = (int)(gridDim.x - 1 - blockIdx.x) * kQBlock;
-    if (q0 >= sq) return;
+    const int wg_q0 = (int)(gridDim.x - 1 - blockIdx.x) * QB * kQBlock;
+    if (wg_q0 >= sq) return;
+    const int q0 = wg_q0 + qb * kQBlock;
+    const bool live = QB == 1 || q0 < sq;   // a trailing wavefront may have no queries: it only helps to fetch
     if (sk <= 0) {
 #pragma unroll
         for (int u = 0; u < kNQ; ++u)
-            if (q0 + 16 * u + n < sq) {
+            if (live && q0 + 16 * u + n < sq) {
                 uint16_t* op = a.out + (int64_t)(q_beg + q0 + 16 * u + n) * a.out_stride0 + (int64_t)head * kD + 4 * g;
                 for (int t = 0; t < 8; ++t) *reinterpret_cast<u32x2*>(op + 16 * t) = u32x2{0u, 0u};
             }
@@ -288,9 +123,13 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         my_q[u] = q0 + 16 * u + n;
         my_limit[u] = a.causal ? (my_q[u] + shift < sk - 1 ? my_q[u] + shift : sk - 1) : sk - 1;
     }
-    const int block_last = q0 + kQBlock - 1 < sq - 1 ? q0 + kQBlock - 1 : sq - 1;
-    const int key_end = a.causal ? (block_last + shift + 1 < sk ? block_last + shift + 1 : sk) : sk;
-    const int nsteps = (key_end + kStep - 1) / kStep;
+    // keys the workgroup walks (its last query block sees the most) and keys this wavefront needs
+    auto key_end_of = [&](int first_q, int count) {
+        const int last = first_q + count - 1 < sq - 1 ? first_q + count - 1 : sq - 1;
+        return a.causal ? (last + shift + 1 < sk ? last + shift + 1 : sk) : sk;
+    };
+    const int nsteps = (key_end_of(wg_q0, QB * kQBlock) + kStep - 1) / kStep;
+    const int my_steps = live ? (key_end_of(q0, kQBlock) + kStep - 1) / kStep : 0;
 
     bf16x8 qreg[kNQ][4];
 #pragma unroll
@@ -316,13 +155,15 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     u32x4 kst[2][kChunks], vst[2][kChunks];
     // chunk i of this thread: row c >> 4 of the tile, 16-byte column c & 15 (both fixed for the kernel)
     int chunk_row[kChunks], chunk_col[kChunks];
+    bool chunk_on[kChunks];
 #pragma unroll
     for (int i = 0; i < kChunks; ++i) {
         const int c = tid + i * kThreads;
-        chunk_row[i] = c >> 4;
+        chunk_on[i] = !kRagged || c < kTileChunks;
+        chunk_row[i] = (c >> 4) & (kStep - 1);
         chunk_col[i] = kvh * kD + (c & 15) * 8;
     }
-    const int tok_stride = (int)a.tok_stride;     // < 2^31 elements (checked on the host)
+    const int tok_stride = (int)a.tok_stride;     // < 2^24 elements (checked on the host)
     auto fetch = [&](auto SLOT, int s) {
         constexpr int S = decltype(SLOT)::value;
         const int tok0 = s * kStep;
@@ -341,6 +182,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         const uint16_t* vp = a.v + base;
 #pragma unroll
         for (int i = 0; i < kChunks; ++i) {
+            if (kRagged && !chunk_on[i]) continue;
             const int r = chunk_row[i] < last ? chunk_row[i] : last;
             const int off = r * tok_stride + chunk_col[i];
             kst[S][i] = load16(kp + off);
@@ -352,6 +194,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         unsigned char* kb = lds_all + buf * kTileBytes;
 #pragma unroll
         for (int i = 0; i < kChunks; ++i) {
+            if (kRagged && !chunk_on[i]) continue;
             const int c = tid + i * kThreads;
             const int row = tile_row(c >> 4);
             *reinterpret_cast<u32x4*>(kb + row * kKRow + (c & 15) * 16) = kst[S][i];
@@ -376,6 +219,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         const unsigned char* vb = kb + kKTileBytes;
         const int tok0 = s * kStep;
 
+        if (QB == 1 || s < my_steps) {   // wavefronts whose queries end earlier skip the keys they cannot see
         // ---- S^T = K Q^T for both query tiles
         f32x4 sc[kNQ][2];
 #pragma unroll
@@ -446,6 +290,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
             for (int u = 0; u < kNQ; ++u)
                 acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pb[u], acc[u][t], 0, 0, 0);
         }
+        }
 
         if (s + 1 < nsteps) stash(NEXT{}, (s + 1) & 1);
         __syncthreads();
@@ -459,6 +304,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         if (s < nsteps) step(S0{}, s);
     }
 
+    if (!live) return;
 #pragma unroll
     for (int u = 0; u < kNQ; ++u) {
         float l = l_run[u] + __shfl_xor(l_run[u], 16);
@@ -477,10 +323,12 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     }
 }
 
-template <int WAVES>
+template <int WAVES, int QB>
 int launch_tiled(const PrefillArgs& a, int64_t max_seqlen_q, int64_t num_seqs, int64_t num_kv_heads, hipStream_t st) {
-    dim3 grid((unsigned)((max_seqlen_q + kQBlock - 1) / kQBlock), (unsigned)num_seqs, (unsigned)num_kv_heads);
-    hipLaunchKernelGGL(paged_prefill_tile_kernel<WAVES>, grid, dim3(64 * WAVES, 1, 1), 2 * kTileBytes, st, a);
+    const int64_t q_per_wg = (int64_t)QB * kQBlock;
+    const int parts = a.group / (WAVES / QB);
+    dim3 grid((unsigned)((max_seqlen_q + q_per_wg - 1) / q_per_wg), (unsigned)num_seqs, (unsigned)(num_kv_heads * parts));
+    hipLaunchKernelGGL((paged_prefill_tile_kernel<WAVES, QB>), grid, dim3(64 * WAVES, 1, 1), 2 * kTileBytes, st, a);
     return (int)hipGetLastError();
 }
 
@@ -503,9 +351,14 @@ extern "C" int infer_paged_prefill_bf16(const void* q, int64_t q_stride0, const 
     if ((q_stride0 | kv_token_stride | out_stride0) & 7) return INFER_KV_EALIGN;
     if (block_table && (kv_block_stride & 7)) return INFER_KV_EALIGN;
     if (kv_token_stride < num_kv_heads * kD || q_stride0 < num_q_heads * kD || out_stride0 < num_q_heads * kD) return INFER_KV_EINVAL;
-    if (num_seqs > 65535 || num_kv_heads > 65535) return INFER_KV_EINVAL;
+    if (num_seqs > 65535 || num_kv_heads * 16 > 65535) return INFER_KV_EINVAL;
     if (kv_token_stride > (1 << 24)) return INFER_KV_EUNSUPPORTED;   // 32-bit offsets inside a tile
     const int G = (int)(num_q_heads / num_kv_heads);
+    // Workgroup shape: the heads of the group (or its largest divisor up to 8) times the number of
+    // consecutive query blocks that brings the workgroup to 4 - 8 wavefronts.
+    int heads = 1;
+    for (int h = G < 8 ? G : 8; h >= 1; --h)
+        if (G % h == 0) { heads = h; break; }
     PrefillArgs a;
     a.q = (const uint16_t*)q; a.q_stride0 = q_stride0;
     a.k = (const uint16_t*)k; a.v = (const uint16_t*)v;
@@ -513,29 +366,20 @@ extern "C" int infer_paged_prefill_bf16(const void* q, int64_t q_stride0, const 
     a.out = (uint16_t*)out; a.out_stride0 = out_stride0;
     a.cu_q = cu_seqlens_q; a.cu_k = cu_seqlens_k;
     a.bt = block_table; a.bt_stride0 = bt_stride0;
-    a.group = G; a.block_size = (int)block_size; a.num_blocks = (int)num_blocks;
-    a.total_k_rows = kv_rows;
+    a.group = G; a.heads_per_wg = heads; a.qblocks_per_wg = heads == 1 ? 4 : (heads <= 3 ? 2 : 1);
+    a.block_size = (int)block_size; a.num_blocks = (int)num_blocks;
     a.scale_log2 = scale * 1.4426950408889634f;
     a.causal = causal ? 1 : 0;
-    switch (G) {   // group sizes with a shared-tile kernel
-        case 1: return launch_tiled<1>(a, max_seqlen_q, num_seqs, num_kv_heads, (hipStream_t)stream);
-        case 2: return launch_tiled<2>(a, max_seqlen_q, num_seqs, num_kv_heads, (hipStream_t)stream);
-        case 4: return launch_tiled<4>(a, max_seqlen_q, num_seqs, num_kv_heads, (hipStream_t)stream);
-        case 8: return launch_tiled<8>(a, max_seqlen_q, num_seqs, num_kv_heads, (hipStream_t)stream);
-        default: break;
+    hipStream_t st = (hipStream_t)stream;
+    switch (heads) {
+        case 1: return launch_tiled<4, 4>(a, max_seqlen_q, num_seqs, num_kv_heads, st);
+        case 2: return launch_tiled<4, 2>(a, max_seqlen_q, num_seqs, num_kv_heads, st);
+        case 3: return launch_tiled<6, 2>(a, max_seqlen_q, num_seqs, num_kv_heads, st);
+        case 4: return launch_tiled<4, 1>(a, max_seqlen_q, num_seqs, num_kv_heads, st);
+        case 5: return launch_tiled<5, 1>(a, max_seqlen_q, num_seqs, num_kv_heads, st);
+        case 6: return launch_tiled<6, 1>(a, max_seqlen_q, num_seqs, num_kv_heads, st);
+        case 7: return launch_tiled<7, 1>(a, max_seqlen_q, num_seqs, num_kv_heads, st);
+        case 8: return launch_tiled<8, 1>(a, max_seqlen_q, num_seqs, num_kv_heads, st);
+        default: return INFER_KV_EUNSUPPORTED;
     }
-    const size_t lds_bytes = (size_t)G * kLdsWave;
-    static bool attr_set[64] = {false};   // the attribute is per device
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
-    if (!attr_set[dev]) {
-        hipError_t e = hipFuncSetAttribute((const void*)paged_prefill_kernel,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 16 * kLdsWave);
-        if (e != hipSuccess) return (int)e;
-        attr_set[dev] = true;
-    }
-    dim3 grid((unsigned)((max_seqlen_q + kQTile - 1) / kQTile), (unsigned)num_seqs, (unsigned)num_kv_heads);
-    dim3 block(64 * G, 1, 1);
-    hipLaunchKernelGGL(paged_prefill_kernel, grid, block, lds_bytes, (hipStream_t)stream, a);
-    return (int)hipGetLastError();
 }

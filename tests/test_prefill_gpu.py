@@ -39,7 +39,7 @@ def test_cfg3_prefix_cached_prefill(gpu):
     assert np.isfinite(f32(out)).all() and err <= ATTN_ATOL
 
 
-@pytest.mark.parametrize("hq,hkv", [(8, 8), (16, 8), (32, 8), (64, 8), (8, 2), (16, 1)])
+@pytest.mark.parametrize("hq,hkv", [(8, 8), (16, 8), (32, 8), (64, 8), (8, 2), (16, 1), (24, 8), (5, 1), (12, 2), (7, 1), (12, 1), (10, 1)])
 def test_small_shapes_with_and_without_prefix(gpu, hq, hkv):
     wl = workloads.make_prefill_workload("p", [1, 15, 16, 17, 33, 300, 257, 600], [0, 0, 0, 0, 0, 256, 256, 512],
                                          hq, hkv, seed=hq + hkv, pad_fraction=0.1).to(gpu)
