@@ -12,7 +12,7 @@
 //   own two 16-row MFMA tiles each.
 // * Weight fragments go from global memory straight into MFMA A-operand registers (16x16x32: lane
 //   (j, g) holds w[row j][k0 + 8 g .. + 7], 16 bytes, 64 contiguous bytes per row and instruction),
-//   two 128-wide K chunks ahead of use; they are never staged.
+//   two 128-wide K chunks ahead of use (a ring of three register slots); they are never staged.
 // * The activations of a chunk ([M, 128], hot in L2) are staged in LDS once per workgroup (double
 //   buffered, 272-byte rows: conflict-free for 16-byte reads of consecutive rows) and read as B
 //   operands; every fragment read feeds both row tiles of the wavefront, which halves the LDS
@@ -81,7 +81,7 @@ __global__ void __launch_bounds__(256) skinny_gemm_kernel(GemmArgs a) {
     }
     const int xs_off = (tid >> 4) * kXRow + (tid & 15) * 16;
 
-    u32x4 wreg[2][kR][4];
+    u32x4 wreg[3][kR][4];
     u32x4 xreg[MT];
     f32x4 acc[kR][MT];
 #pragma unroll
@@ -107,53 +107,52 @@ __global__ void __launch_bounds__(256) skinny_gemm_kernel(GemmArgs a) {
         for (int i = 0; i < MT; ++i) *reinterpret_cast<u32x4*>(&xs[buf][xs_off + 16 * i * kXRow]) = xreg[i];
     };
     // B fragment of batch tile t at K step kk: lane (j, g) reads x[16 t + j][32 kk + 8 g .. + 7].
-    // The fragments of the next K step are read from LDS while the MFMAs of this one run.
     auto compute = [&](auto SLOT, int buf) {
         constexpr int slot = decltype(SLOT)::value;
         const unsigned char* xb = &xs[buf][j * kXRow + 16 * g];
-        u32x4 frag[2][MT];
-#pragma unroll
-        for (int t = 0; t < MT; ++t) frag[0][t] = *reinterpret_cast<const u32x4*>(xb + 16 * t * kXRow);
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
-            if (kk < 3) {
+            u32x4 frag[MT];
 #pragma unroll
-                for (int t = 0; t < MT; ++t)
-                    frag[(kk + 1) & 1][t] = *reinterpret_cast<const u32x4*>(xb + 16 * t * kXRow + 64 * (kk + 1));
-            }
-            __builtin_amdgcn_sched_barrier(0);      // keep the reads of the next step ahead of these MFMAs
+            for (int t = 0; t < MT; ++t) frag[t] = *reinterpret_cast<const u32x4*>(xb + 16 * t * kXRow + 64 * kk);
+            __builtin_amdgcn_sched_barrier(0);      // all reads of the step first, then its MFMAs
 #pragma unroll
             for (int t = 0; t < MT; ++t)
 #pragma unroll
                 for (int r = 0; r < kR; ++r)
                     acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wreg[slot][r][kk]),
-                                                                        as_bf16x8(frag[kk & 1][t]), acc[r][t], 0, 0, 0);
+                                                                        as_bf16x8(frag[t]), acc[r][t], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
 
-    // chunk c: weights in register slot c & 1, activations in LDS buffer c & 1
+    // chunk c: weights in ring slot c % 3, activations in LDS buffer c & 1.  The loads of chunk c + 2
+    // are issued before chunk c is consumed, so two chunks (16 KiB per wavefront) stay in flight
+    // while the MFMAs run: memory latency, not LDS latency, is what has to be hidden.
     using R0 = std::integral_constant<int, 0>;
     using R1 = std::integral_constant<int, 1>;
+    using R2 = std::integral_constant<int, 2>;
     issue_x(0);
     issue_w(R0{}, 0);
     issue_w(R1{}, 1);
     park_x(0);
     issue_x(1);
     __syncthreads();
-    auto step = [&](auto SLOT, int c) {
+    auto step = [&](auto SLOT, auto AHEAD, int c) {
+        issue_w(AHEAD, c + 2);         // into the slot chunk c - 1 has left
         compute(SLOT, c & 1);
         park_x((c + 1) & 1);           // the buffer chunk c - 1 was read from; all waves are past it
         issue_x(c + 2);
-        issue_w(SLOT, c + 2);
         __syncthreads();
     };
     int c = 0;
-    for (; c + 1 < a.chunks; c += 2) {
-        step(R0{}, c);
-        step(R1{}, c + 1);
+    for (; c + 2 < a.chunks; c += 3) {
+        step(R0{}, R2{}, c);
+        step(R1{}, R0{}, c + 1);
+        step(R2{}, R1{}, c + 2);
     }
-    if (c < a.chunks) step(R0{}, c);
+    if (c < a.chunks) step(R0{}, R2{}, c);
+    if (c + 1 < a.chunks) step(R1{}, R0{}, c + 1);
 
     // accumulator element e of lane (j, g) in tile (r, t) is y[16 t + j][n0 + 16 r + 4 g + e]
 #pragma unroll
