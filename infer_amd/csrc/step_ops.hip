@@ -62,6 +62,13 @@ __global__ void __launch_bounds__(kNormThreads) rms_norm_kernel(NormArgs a) {
     const uint16_t* xr = a.x + row * a.x_stride0;
     uint16_t* rr = a.residual ? a.residual + row * a.residual_stride0 : nullptr;
 
+    // the weights do not depend on the reduction: fetch them with the first round of loads
+    u32x4 wv[kNormMaxChunks];
+#pragma unroll
+    for (int j = 0; j < kNormMaxChunks; ++j) {
+        const int c = tid + j * kNormThreads;
+        if (c < a.chunks) wv[j] = *reinterpret_cast<const u32x4*>(a.weight + 8 * c);
+    }
     float v[kNormMaxChunks][8];
     float ss = 0.f;
 #pragma unroll
@@ -109,7 +116,7 @@ __global__ void __launch_bounds__(kNormThreads) rms_norm_kernel(NormArgs a) {
         const int c = tid + j * kNormThreads;
         if (c < a.chunks) {
             float w[8], o[8];
-            unpack8(*reinterpret_cast<const u32x4*>(a.weight + 8 * c), w);
+            unpack8(wv[j], w);
 #pragma unroll
             for (int e = 0; e < 8; ++e) o[e] = rb(v[j][e] * rs) * w[e];
             *reinterpret_cast<u32x4*>(orow + 8 * c) = pack8(o);
