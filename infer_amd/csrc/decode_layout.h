@@ -10,7 +10,7 @@
 #define INFER_KV_MAX_SPLIT_WG 1024
 
 struct DecodeWorkspace {
-    size_t header_off;      // int32[64]: {workgroups, steps per span, total steps}
+    size_t header_off;      // int32[64]: {spans used by the last launch, total steps} (diagnostic)
     size_t seg_first_off;   // int32[batch]: first split workgroup that touched the sequence
     size_t seg_last_off;    // int32[batch]: last one
     size_t rec_off;         // [slots] records of rec_stride bytes, one per (segment, KV head)

@@ -429,13 +429,34 @@ __global__ void __launch_bounds__(512) paged_decode_split_kernel(DecodeArgs a) {
     // Equal shares: the first `rem` workgroups take one step more.  With fewer steps than workgroups
     // every step gets a workgroup of its own: on tiny problems a longer span would only serialise
     // memory latency (measured: one sequence of 512 tokens 14.7 -> 6.7 us).
-    const int q = total / W, rem = total - q * W;
-    const int lo = w * q + (w < rem ? w : rem);
-    const int hi = lo + q + (w < rem ? 1 : 0);
+    //
+    // The share is a whole number of steps, so with `rem` left over most workgroups idle for the
+    // last step of the launch (64 sequences of about 2450 tokens: 4906 steps over 256 workgroups = 19 each and 42 with 20, i.e.
+    // 214 compute units wait out a twentieth of the run).  Each lane therefore tries one span
+    // count in (3W/4, W] and the wave keeps the one whose rounded-up shares waste the fewest steps
+    // (ties: the larger count); the workgroups beyond it leave at once.  Bandwidth is flat over
+    // that range of resident workgroups, so the shorter tail is a pure gain.
+    int spans = W;
+    if (total > W && W >= 4) {
+        const int cand = W - lane;
+        const bool ok = lane < W / 4;
+        const int share = ok ? (total + cand - 1) / cand : 0;
+        int key = ok ? ((share * cand - total) << 7) | lane : 0x7fffffff;   // lane < 64 < 128
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const int other = __shfl_xor(key, o);
+            key = other < key ? other : key;
+        }
+        spans = W - (__builtin_amdgcn_readfirstlane(key) & 127);
+    }
     if (w == 0 && h == 0 && lane == 0) {
-        a.header[0] = W;
+        a.header[0] = spans;
         a.header[1] = total;
     }
+    if (w >= spans) return;
+    const int q = total / spans, rem = total - q * spans;
+    const int lo = w * q + (w < rem ? w : rem);
+    const int hi = lo + q + (w < rem ? 1 : 0);
     if (lo >= hi) return;
 
     int nseg = 0, nord = 0, nsteps = 0, tblv = 0;
