@@ -144,10 +144,13 @@ class Sampler(nn.Module):
     softmax by the exponential-race trick."""
 
     def forward(self, logits: torch.Tensor, temperatures: torch.Tensor, all_greedy: bool = False) -> torch.Tensor:
+        if all_greedy:
+            # The caller knows on the host that every temperature is 0.  Widening bf16 to float is exact
+            # and order-preserving and argmax breaks ties by the lower index in either type, so the
+            # float copy of the [batch, vocab] logits (0.4 ms per decode step at batch 128) is skipped.
+            return logits.argmax(dim=-1)
         logits = logits.to(torch.float)
         greedy_tokens = logits.argmax(dim=-1)
-        if all_greedy:      # the caller knows on the host that every temperature is 0
-            return greedy_tokens
         logits.div_(temperatures.unsqueeze(dim=1))
         probs = torch.softmax(logits, dim=-1, dtype=torch.float)
         sample_tokens = probs.div_(torch.empty_like(probs).exponential_(1) + 1e-10).argmax(dim=-1)

@@ -204,6 +204,11 @@ def test_sampler_temperature(gpu):
     temps = torch.tensor([0.0, 1.0, 0.5, 0.0], device=gpu)
     assert Sampler()(logits, temps).tolist() == [7, 7, 7, 7]
     assert Sampler()(logits, temps * 0, all_greedy=True).tolist() == [7, 7, 7, 7]
+    # the all-greedy shortcut works on the bf16 logits: same tokens as the float path, ties included
+    coarse = (torch.randn((64, 50000), device=gpu) * 4).round().to(torch.bfloat16)   # many exact ties
+    zeros = torch.zeros(64, device=gpu)
+    assert torch.equal(Sampler()(coarse, zeros, all_greedy=True), Sampler()(coarse, zeros))
+    assert torch.equal(Sampler()(coarse, zeros, all_greedy=True), coarse.float().argmax(dim=-1))
     flat = torch.zeros((2000, 4), device=gpu)
     draws = Sampler()(flat, torch.ones(2000, device=gpu))
     counts = torch.bincount(draws, minlength=4).float() / 2000
