@@ -93,6 +93,21 @@ __device__ __forceinline__ int wave_inclusive_scan(int x, int lane) {
     return x;
 }
 
+// max over lanes l and l ^ 16 (l ^ 32) in every lane.  v_permlane16_swap exchanges the odd 16-lane rows
+// of its first operand with the even rows of its second: fed the same value twice it returns
+// (rows 0 0 2 2, rows 1 1 3 3), whose maximum is the reduction; v_permlane32_swap does the same with
+// the two halves of the wavefront.  Both stay on the vector pipe, where a shuffle would go through LDS.
+__device__ __forceinline__ float max_xor16(float x) {
+    const unsigned u = __builtin_bit_cast(unsigned, x);
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+}
+__device__ __forceinline__ float max_xor32(float x) {
+    const unsigned u = __builtin_bit_cast(unsigned, x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+}
+
 // Keeps the compiler from moving LDS traffic across this point.  The LDS queue of one
 // wavefront is processed in order, so within a wavefront a compiler barrier is all the
 // write -> read -> write sequence on the private tile needs.
@@ -328,8 +343,7 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
         float mx = sv[0];
 #pragma unroll
         for (int i = 1; i < 8; ++i) mx = fmaxf(mx, sv[i]);
-        mx = fmaxf(mx, __shfl_xor(mx, 16));
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        mx = max_xor32(max_xor16(mx));
         const float m_new = fmaxf(m_run, mx);
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
         m_run = m_new;

@@ -64,6 +64,22 @@ __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 x) { return __builtin_bit_cast
 __device__ __forceinline__ u32x4 load16(const uint16_t* p) { return *reinterpret_cast<const u32x4*>(p); }
 __device__ __forceinline__ void lds_order() { __asm__ volatile("" ::: "memory"); }
 
+// max over lanes l and l ^ 16 (l ^ 32) in every lane.  v_permlane16_swap exchanges the odd 16-lane rows
+// of its first operand with the even rows of its second: fed the same value twice it returns
+// (rows 0 0 2 2, rows 1 1 3 3), whose maximum is the reduction; v_permlane32_swap does the same with
+// the two halves of the wavefront.  Both run on the vector pipe: a shuffle through LDS
+// (ds_bpermute) would put two LDS round trips on the critical path of every softmax.
+__device__ __forceinline__ float max_xor16(float x) {
+    const unsigned u = __builtin_bit_cast(unsigned, x);
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+}
+__device__ __forceinline__ float max_xor32(float x) {
+    const unsigned u = __builtin_bit_cast(unsigned, x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+}
+
 // LDS layout of a tile: key k of the step sits in row  16 ((k >> 2) & 1) + 4 (k >> 3) + (k & 3),  so
 // that the 16 K rows one ds_read_b128 pass touches (one MFMA row tile) and the 8 V rows one
 // transposing read pass touches are consecutive rows.  With a row stride of 272 B (68 banks:
@@ -256,8 +272,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
             float mx = sv[0];
 #pragma unroll
             for (int i = 1; i < 8; ++i) mx = fmaxf(mx, sv[i]);
-            mx = fmaxf(mx, __shfl_xor(mx, 16));
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            mx = max_xor32(max_xor16(mx));
             mx *= a.scale_log2;                                  // scale > 0: the maximum commutes with it
             const bool grow = mx > m_run[u] + kLazy;             // -inf + kLazy = -inf: the first finite maximum always grows
             if (__any(grow)) {
