@@ -139,6 +139,10 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         my_q[u] = q0 + 16 * u + n;
         my_limit[u] = a.causal ? (my_q[u] + shift < sk - 1 ? my_q[u] + shift : sk - 1) : sk - 1;
     }
+    // lane 0 holds the earliest query of a tile, hence the smallest limit
+    int lim_lo[kNQ];
+#pragma unroll
+    for (int u = 0; u < kNQ; ++u) lim_lo[u] = __builtin_amdgcn_readfirstlane(my_limit[u]);
     // keys the workgroup walks (its last query block sees the most) and keys this wavefront needs
     auto key_end_of = [&](int first_q, int count) {
         const int last = first_q + count - 1 < sq - 1 ? first_q + count - 1 : sq - 1;
@@ -148,6 +152,9 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     const int my_steps = live ? (key_end_of(q0, kQBlock) + kStep - 1) / kStep : 0;
 
     bf16x8 qreg[kNQ][4];
+    bf16x8 ones;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ones[i] = (__bf16)1.0f;
 #pragma unroll
     for (int u = 0; u < kNQ; ++u) {
         const u32x4 z = {0u, 0u, 0u, 0u};
@@ -157,13 +164,17 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         for (int j = 0; j < 4; ++j) qreg[u][j] = as_bf16x8(live ? load16(qp + 32 * j) : z);
     }
     f32x4 acc[kNQ][8];
-    float m_run[kNQ], l_run[kNQ];
+    // Row sums ride the matrix pipe: ones[16 x 32] . P^T adds the 32 probabilities of a step for every
+    // query (one MFMA per tile and step instead of eight vector adds), of the same bf16 values the
+    // numerator is built from; all four accumulator rows of a lane hold the same sum.
+    f32x4 lacc[kNQ];
+    float m_run[kNQ];
 #pragma unroll
     for (int u = 0; u < kNQ; ++u) {
 #pragma unroll
         for (int t = 0; t < 8; ++t) acc[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
         m_run[u] = -INFINITY;
-        l_run[u] = 0.f;
+        lacc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
     // cooperative tile fetch: chunk c covers bytes [16 (c % 16), +16) of row c / 16
@@ -180,29 +191,64 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         chunk_col[i] = kvh * kD + (c & 15) * 8;
     }
     const int tok_stride = (int)a.tok_stride;     // < 2^24 elements (checked on the host)
+    uint32_t chunk_off[kChunks];                  // element offset of the chunk inside a tile
+#pragma unroll
+    for (int i = 0; i < kChunks; ++i) chunk_off[i] = (uint32_t)(chunk_row[i] * tok_stride + chunk_col[i]);
+    // The block ids of the sequence sit in two registers (lane i: blocks i and 64 + i), read with
+    // v_readlane: a table lookup in memory, behind a division by the block size, would put some
+    // 300 ns of dependent scalar work in front of every tile fetch.  Tiles are fetched in order, so
+    // the block index and the step inside the block are counters.
+    const int steps_per_blk = a.block_size / kStep;
+    int tbl0 = 0, tbl1 = 0;
+    if (a.bt) {
+        const int nblk = (nsteps + steps_per_blk - 1) / steps_per_blk;
+        const int32_t* row = a.bt + (int64_t)b * a.bt_stride0;
+        if (lane < nblk) tbl0 = row[lane];
+        if (64 + lane < nblk) tbl1 = row[64 + lane];
+    }
+    int f_blk = 0, f_in = 0;      // block index and step inside it of the next tile to fetch
+    int64_t f_base = 0;           // element offset of that block
     auto fetch = [&](auto SLOT, int s) {
         constexpr int S = decltype(SLOT)::value;
         const int tok0 = s * kStep;
         int64_t base;
         if (a.bt) {
-            int blk = __builtin_amdgcn_readfirstlane(a.bt[(int64_t)b * a.bt_stride0 + tok0 / a.block_size]);
-            blk = blk < 0 ? 0 : (blk >= a.num_blocks ? a.num_blocks - 1 : blk);
-            base = (int64_t)blk * a.blk_stride + (int64_t)(tok0 % a.block_size) * a.tok_stride;
+            if (f_in == 0) {
+                int blk;
+                if (f_blk < 64) blk = __builtin_amdgcn_readlane(tbl0, f_blk);
+                else if (f_blk < 128) blk = __builtin_amdgcn_readlane(tbl1, f_blk - 64);
+                else blk = __builtin_amdgcn_readfirstlane(a.bt[(int64_t)b * a.bt_stride0 + f_blk]);
+                blk = blk < 0 ? 0 : (blk >= a.num_blocks ? a.num_blocks - 1 : blk);
+                f_base = (int64_t)blk * a.blk_stride;
+            }
+            base = f_base + (int64_t)(f_in * kStep) * a.tok_stride;
+            if (++f_in == steps_per_blk) { f_in = 0; ++f_blk; }
         } else {
             base = ((int64_t)k_beg + tok0) * a.tok_stride;
         }
-        // rows past the end of the sequence (last step only) re-read its last row: finite data whose
-        // probabilities are masked to zero, instead of whatever lies behind the sequence
-        const int last = sk - 1 - tok0;
         const uint16_t* kp = a.k + base;
         const uint16_t* vp = a.v + base;
+        if (tok0 + kStep <= sk) {
+            // whole tile inside the sequence: uniform base + the thread's constant 32-bit offset, no
+            // address arithmetic on the vector pipe
 #pragma unroll
-        for (int i = 0; i < kChunks; ++i) {
-            if (kRagged && !chunk_on[i]) continue;
-            const int r = chunk_row[i] < last ? chunk_row[i] : last;
-            const int off = r * tok_stride + chunk_col[i];
-            kst[S][i] = load16(kp + off);
-            vst[S][i] = load16(vp + off);
+            for (int i = 0; i < kChunks; ++i) {
+                if (kRagged && !chunk_on[i]) continue;
+                kst[S][i] = load16(kp + chunk_off[i]);
+                vst[S][i] = load16(vp + chunk_off[i]);
+            }
+        } else {
+            // rows past the end of the sequence (last step only) re-read its last row: finite data whose
+            // probabilities are masked to zero, instead of whatever lies behind the sequence
+            const int last = sk - 1 - tok0;
+#pragma unroll
+            for (int i = 0; i < kChunks; ++i) {
+                if (kRagged && !chunk_on[i]) continue;
+                const int r = chunk_row[i] < last ? chunk_row[i] : last;
+                const uint32_t off = (uint32_t)(r * tok_stride + chunk_col[i]);
+                kst[S][i] = load16(kp + off);
+                vst[S][i] = load16(vp + off);
+            }
         }
     };
     auto stash = [&](auto SLOT, int buf) {
@@ -264,7 +310,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) sv[4 * t + e] = sc[u][t][e];
-            if (tok0 + kStep - 1 > my_limit[u]) {
+            if (tok0 + kStep - 1 > lim_lo[u]) {      // wave-uniform: off the diagonal no lane masks anything
 #pragma unroll
                 for (int i = 0; i < 8; ++i)
                     if (tok0 + 8 * g + i > my_limit[u]) sv[i] = -INFINITY;
@@ -278,19 +324,15 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
             if (__any(grow)) {
                 const float alpha = grow ? __builtin_amdgcn_exp2f(m_run[u] - mx) : 1.f;
                 m_run[u] = grow ? mx : m_run[u];
-                l_run[u] *= alpha;
+                lacc[u] *= alpha;
 #pragma unroll
                 for (int t = 0; t < 8; ++t) acc[u][t] *= alpha;
             }
             const float m_neg = m_run[u] == -INFINITY ? 0.f : -m_run[u];
-            float psum = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[i], a.scale_log2, m_neg));
-                psum += p;
-                pb[u][i] = (__bf16)p;
-            }
-            l_run[u] += psum;
+            for (int i = 0; i < 8; ++i)
+                pb[u][i] = (__bf16)__builtin_amdgcn_exp2f(__builtin_fmaf(sv[i], a.scale_log2, m_neg));
+            lacc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb[u], lacc[u], 0, 0, 0);
         }
 
         // ---- O^T += V^T P^T, every V fragment used for both query tiles
@@ -307,7 +349,10 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         }
         }
 
-        if (s + 1 < nsteps) stash(NEXT{}, (s + 1) & 1);
+        // Unconditional: after the last step this parks stale registers in a buffer nobody reads again,
+        // and in exchange every path through the loop has waited for this slot's loads, so the fetch
+        // into it at the top of the next step needs no wait that would also drain the newest loads.
+        stash(NEXT{}, (s + 1) & 1);
         __syncthreads();
     };
     {
@@ -322,8 +367,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     if (!live) return;
 #pragma unroll
     for (int u = 0; u < kNQ; ++u) {
-        float l = l_run[u] + __shfl_xor(l_run[u], 16);
-        l += __shfl_xor(l, 32);
+        const float l = lacc[u][0];
         if (my_q[u] < sq) {
             const float inv = l > 0.f ? 1.f / l : 0.f;
             uint16_t* op = a.out + (int64_t)(q_beg + my_q[u]) * a.out_stride0 + (int64_t)head * kD + 4 * g;
