@@ -15,9 +15,10 @@
 // A workgroup is 4 to 8 wavefronts that read the same keys: the query heads of one KV head (all of
 // them, or a divisor-sized part when the group is larger than 8) times as many consecutive query
 // blocks as fit (4 blocks for a group of 1, 2 for groups of 2 and 3, 1 otherwise).  They share
-// every 32-key K tile and V tile through LDS: the tiles are fetched once per workgroup with fully
-// coalesced 16-byte loads and double-buffered (the loads of tile s + 2 are in flight in registers
-// while tile s + 1 sits in LDS and tile s is consumed; one barrier per step).
+// every 32-key K tile and V tile through LDS: the tiles are fetched once per workgroup, straight
+// from global memory into a ring of three LDS buffers (global_load_dwordx4 ... lds: no registers, no
+// LDS store instructions; tile s + 2 is in flight while tile s + 1 has landed and tile s is consumed;
+// one barrier per step).  Without staging registers the kernel fits three wavefronts per SIMD.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -82,28 +83,28 @@ __device__ __forceinline__ float max_xor32(float x) {
 
 // LDS layout of a tile: key k of the step sits in row  16 ((k >> 2) & 1) + 4 (k >> 3) + (k & 3),  so
 // that the 16 K rows one ds_read_b128 pass touches (one MFMA row tile) and the 8 V rows one
-// transposing read pass touches are consecutive rows.  With a row stride of 272 B (68 banks:
-// consecutive rows start 4 banks apart) both read patterns run at the full LDS rate (measured with
-// a probe: 256 B rows cost 4x, 288 B rows 1.2x); the 16-byte stores of a row cover all banks anyway.
+// transposing read pass touches are consecutive rows.  Rows are 256 B (no padding: the tiles are
+// written by global_load ... lds, which fills 1 KiB = four whole rows per wavefront instruction)
+// and the sixteen 16-byte chunks of row r are rotated by r positions (chunk c sits at position
+// (c + r) % 16), which spreads consecutive rows over the banks exactly like a 272-byte row stride
+// does (measured with a probe: plain 256 B rows cost 4x on both read patterns).
 constexpr int kNQ = 2;
 constexpr float kLazy = 8.f;
 constexpr int kQBlock = kNQ * kQTile;
-constexpr int kKRow = 272;
-constexpr int kVRow = 272;
-constexpr int kKTileBytes = kStep * kKRow;
-constexpr int kVTileBytes = kStep * kVRow;
+constexpr int kRowB = 256;
+constexpr int kKTileBytes = kStep * kRowB;
+constexpr int kVTileBytes = kStep * kRowB;
 constexpr int kTileBytes = kKTileBytes + kVTileBytes;     // one K tile + one V tile
+constexpr int kRing = 3;                                  // tiles resident in LDS: consumed, landed, in flight
+constexpr int kTblLds = 512;                              // block ids of a sequence kept in LDS
 __device__ __forceinline__ int tile_row(int k) { return 16 * ((k >> 2) & 1) + 4 * (k >> 3) + (k & 3); }
+__device__ __forceinline__ int tile_key(int r) { return (((r >> 2) & 3) << 3) | ((r >> 4) << 2) | (r & 3); }   // inverse of tile_row
 
 // WAVES = heads per workgroup x QB, QB = query blocks per workgroup (a compile-time constant so that the
 // common QB == 1 case carries no per-wavefront step guard).
 template <int WAVES, int QB>
-__global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) paged_prefill_tile_kernel(PrefillArgs a) {
+__global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3, 3))) paged_prefill_tile_kernel(PrefillArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_all[];   // [2][K tile | V tile]
-    constexpr int kThreads = 64 * WAVES;
-    constexpr int kTileChunks = kStep * 16;                            // 16-byte chunks of a 32 x 256 B tile
-    constexpr int kChunks = (kTileChunks + kThreads - 1) / kThreads;   // tile chunks per thread
-    constexpr bool kRagged = kTileChunks % kThreads != 0;              // the last round is only partly used
     constexpr int kHeads = WAVES / QB;                                 // query heads per workgroup
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -177,47 +178,67 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         lacc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    // cooperative tile fetch: chunk c covers bytes [16 (c % 16), +16) of row c / 16
-    // two tiles are in flight in registers (slots 0 and 1 alternate), a third is being consumed from LDS
-    u32x4 kst[2][kChunks], vst[2][kChunks];
-    // chunk i of this thread: row c >> 4 of the tile, 16-byte column c & 15 (both fixed for the kernel)
-    int chunk_row[kChunks], chunk_col[kChunks];
-    bool chunk_on[kChunks];
-#pragma unroll
-    for (int i = 0; i < kChunks; ++i) {
-        const int c = tid + i * kThreads;
-        chunk_on[i] = !kRagged || c < kTileChunks;
-        chunk_row[i] = (c >> 4) & (kStep - 1);
-        chunk_col[i] = kvh * kD + (c & 15) * 8;
-    }
+    // Cooperative tile fetch, global memory -> LDS without passing through registers.  One
+    // global_load_dwordx4 ... lds of a wavefront fills 1 KiB of LDS, lane l at byte 16 l: four rows
+    // of a tile, lane l = chunk position l % 16 of row l / 16, which by the rotation above is chunk
+    // (l % 16 - row) % 16 of that row's key.  A tile pair is 16 such loads (8 K, 8 V); wavefront w
+    // issues loads w, w + WAVES, ...  Every wavefront issues the same number per tile (a surplus
+    // one repeats load 0: same bytes to the same place), so "this tile has landed" is a fixed count
+    // of its own outstanding loads followed by the workgroup barrier.
+    //
+    // The load is issued as inline assembly on purpose.  Through the compiler's builtin every later
+    // LDS read is preceded by a wait for ALL outstanding loads (the compiler cannot see that a read
+    // touches another ring buffer than the one being filled), which would leave the newest tile half a
+    // step to arrive instead of two.  Here the waits are the explicit counts below.  M0 (the LDS base
+    // of the transfer) is put back afterwards.
+    typedef __attribute__((address_space(3))) void* lptr_t;
+    auto dma16 = [&](const uint16_t* src, unsigned char* dst) {
+        const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)dst;
+        uint32_t keep;
+        __asm__ volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
+                         : "=&s"(keep) : "v"(src), "s"(lds_addr) : "memory");
+    };
+    constexpr int kLoads = (16 + WAVES - 1) / WAVES;
     const int tok_stride = (int)a.tok_stride;     // < 2^24 elements (checked on the host)
-    uint32_t chunk_off[kChunks];                  // element offset of the chunk inside a tile
+    uint32_t ld_off[kLoads];                      // element offset inside a tile of what this lane fetches
+    int ld_dst[kLoads];                           // LDS byte offset of the load inside a tile pair (uniform)
+    auto ld_key = [&](int i) {                    // key (row of the tile in memory) of load i of this lane
+        const int L = wave + i * WAVES < 16 ? wave + i * WAVES : 0;
+        return tile_key(4 * (L & 7) + (lane >> 4));
+    };
+    auto ld_col = [&](int i) {                    // its element column
+        const int L = wave + i * WAVES < 16 ? wave + i * WAVES : 0;
+        return (uint32_t)(kvh * kD + (((lane & 15) - (4 * (L & 7) + (lane >> 4))) & 15) * 8);
+    };
 #pragma unroll
-    for (int i = 0; i < kChunks; ++i) chunk_off[i] = (uint32_t)(chunk_row[i] * tok_stride + chunk_col[i]);
-    // The block ids of the sequence sit in two registers (lane i: blocks i and 64 + i), read with
-    // v_readlane: a table lookup in memory, behind a division by the block size, would put some
-    // 300 ns of dependent scalar work in front of every tile fetch.  Tiles are fetched in order, so
-    // the block index and the step inside the block are counters.
+    for (int i = 0; i < kLoads; ++i) {
+        const int L = wave + i * WAVES < 16 ? wave + i * WAVES : 0;
+        ld_off[i] = (uint32_t)(ld_key(i) * tok_stride) + ld_col(i);
+        ld_dst[i] = (L >> 3) * kKTileBytes + (L & 7) * 1024;
+    }
+    // The first kTblLds block ids of the sequence are copied to LDS behind the ring (one barrier, before
+    // anything is fetched): a lookup in memory, behind a division by the block size, would put some
+    // 300 ns of dependent work in front of every tile fetch, and a register copy gets spilled, whose
+    // reload is a vector load and so drains the ring.  Tiles are fetched in order, so the block index
+    // and the step inside the block are counters.
     const int steps_per_blk = a.block_size / kStep;
-    int tbl0 = 0, tbl1 = 0;
+    int* lds_tbl = reinterpret_cast<int*>(lds_all + kRing * kTileBytes);
     if (a.bt) {
         const int nblk = (nsteps + steps_per_blk - 1) / steps_per_blk;
         const int32_t* row = a.bt + (int64_t)b * a.bt_stride0;
-        if (lane < nblk) tbl0 = row[lane];
-        if (64 + lane < nblk) tbl1 = row[64 + lane];
+        for (int i = tid; i < nblk && i < kTblLds; i += 64 * WAVES) lds_tbl[i] = row[i];
+        __syncthreads();
     }
     int f_blk = 0, f_in = 0;      // block index and step inside it of the next tile to fetch
     int64_t f_base = 0;           // element offset of that block
-    auto fetch = [&](auto SLOT, int s) {
-        constexpr int S = decltype(SLOT)::value;
+    auto fetch = [&](int s, int buf) {
         const int tok0 = s * kStep;
         int64_t base;
         if (a.bt) {
             if (f_in == 0) {
                 int blk;
-                if (f_blk < 64) blk = __builtin_amdgcn_readlane(tbl0, f_blk);
-                else if (f_blk < 128) blk = __builtin_amdgcn_readlane(tbl1, f_blk - 64);
-                else blk = __builtin_amdgcn_readfirstlane(a.bt[(int64_t)b * a.bt_stride0 + f_blk]);
+                if (f_blk < kTblLds) blk = __builtin_amdgcn_readfirstlane(lds_tbl[f_blk]);
+                else blk = __builtin_amdgcn_readfirstlane(a.bt[(int64_t)b * a.bt_stride0 + f_blk]);   // drains the ring
                 blk = blk < 0 ? 0 : (blk >= a.num_blocks ? a.num_blocks - 1 : blk);
                 f_base = (int64_t)blk * a.blk_stride;
             }
@@ -228,57 +249,57 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         }
         const uint16_t* kp = a.k + base;
         const uint16_t* vp = a.v + base;
+        unsigned char* dst = lds_all + buf * kTileBytes;
         if (tok0 + kStep <= sk) {
-            // whole tile inside the sequence: uniform base + the thread's constant 32-bit offset, no
-            // address arithmetic on the vector pipe
 #pragma unroll
-            for (int i = 0; i < kChunks; ++i) {
-                if (kRagged && !chunk_on[i]) continue;
-                kst[S][i] = load16(kp + chunk_off[i]);
-                vst[S][i] = load16(vp + chunk_off[i]);
+            for (int i = 0; i < kLoads; ++i) {
+                const uint16_t* src = (ld_dst[i] < kKTileBytes ? kp : vp) + ld_off[i];
+                dma16(src, dst + ld_dst[i]);
             }
         } else {
             // rows past the end of the sequence (last step only) re-read its last row: finite data whose
             // probabilities are masked to zero, instead of whatever lies behind the sequence
             const int last = sk - 1 - tok0;
 #pragma unroll
-            for (int i = 0; i < kChunks; ++i) {
-                if (kRagged && !chunk_on[i]) continue;
-                const int r = chunk_row[i] < last ? chunk_row[i] : last;
-                const uint32_t off = (uint32_t)(r * tok_stride + chunk_col[i]);
-                kst[S][i] = load16(kp + off);
-                vst[S][i] = load16(vp + off);
+            for (int i = 0; i < kLoads; ++i) {
+                const int r = ld_key(i) < last ? ld_key(i) : last;
+                const uint16_t* src = (ld_dst[i] < kKTileBytes ? kp : vp) + ((uint32_t)(r * tok_stride) + ld_col(i));
+                dma16(src, dst + ld_dst[i]);
             }
         }
     };
-    auto stash = [&](auto SLOT, int buf) {
-        constexpr int S = decltype(SLOT)::value;
-        unsigned char* kb = lds_all + buf * kTileBytes;
-#pragma unroll
-        for (int i = 0; i < kChunks; ++i) {
-            if (kRagged && !chunk_on[i]) continue;
-            const int c = tid + i * kThreads;
-            const int row = tile_row(c >> 4);
-            *reinterpret_cast<u32x4*>(kb + row * kKRow + (c & 15) * 16) = kst[S][i];
-            *reinterpret_cast<u32x4*>(kb + kKTileBytes + row * kVRow + (c & 15) * 16) = vst[S][i];
-        }
-    };
-    using S0 = std::integral_constant<int, 0>;
-    using S1 = std::integral_constant<int, 1>;
+    // this wavefront's loads of all tiles but the newest have landed / of all tiles have landed
+    auto landed_but_newest = [&]() { __builtin_amdgcn_s_waitcnt(0x0F70 | kLoads); };
+    auto landed_all = [&]() { __builtin_amdgcn_s_waitcnt(0x0F70); };
 
-    // tile s travels in slot s % 2: fetched during step s - 2, stored to LDS at the end of step s - 1
-    fetch(S0{}, 0);
-    if (nsteps > 1) fetch(S1{}, 1);
-    stash(S0{}, 0);
+    // Read addresses under the rotation.  K operand row n of MFMA row tile t is key
+    // 8 (n / 4) + 4 t + n % 4 = LDS row 16 t + n, K step j is chunk 4 j + g of it; V keys 8 g + n / 4 (lo)
+    // and 8 g + 4 + n / 4 (hi) sit in LDS rows 4 g + n / 4 and 16 more, columns 16 t + 4 (n % 4) .. + 3 are
+    // half n % 2 of chunk 2 t + (n % 4) / 2.  A row 16 further down has the same rotation.
+    int k_addr[4], v_addr[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) k_addr[j] = n * kRowB + (((4 * j + g + n) & 15) << 4);
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        const int row = 4 * g + (n >> 2);
+        v_addr[t] = kKTileBytes + row * kRowB + (((2 * t + ((n & 3) >> 1) + row) & 15) << 4) + (n & 1) * 8;
+    }
+
+    // tile s lives in ring buffer s % 3: requested at the top of step s - 2, landed (own loads counted,
+    // then the barrier) at the end of step s - 1, read during step s; the buffer is requested again at
+    // the top of step s + 1, after the barrier that ends step s.
+    // Q and the block ids have arrived before the first transfer is issued: the compiler does not see
+    // the transfers, so any wait of its own for these earlier loads inside the loop would be a wait for
+    // zero outstanding loads and drain the ring.
+    landed_all();
+    fetch(0, 0);
+    if (nsteps > 1) { fetch(1, 1); landed_but_newest(); } else { landed_all(); }
     __syncthreads();
 
-    // K operand row n of MFMA row tile t is key 8 (n / 4) + 4 t + n % 4, which sits in LDS row 16 t + n
-    auto step = [&](auto SLOT, int s) {
-        constexpr int S = decltype(SLOT)::value;          // slot of tile s (just consumed from LDS): free again
-        using NEXT = std::integral_constant<int, 1 - S>;  // slot of tile s + 1
-        if (s + 2 < nsteps) fetch(SLOT, s + 2);
-        const unsigned char* kb = lds_all + (s & 1) * kTileBytes;
-        const unsigned char* vb = kb + kKTileBytes;
+    auto step = [&](int s, int buf) {
+        const int buf2 = buf == 0 ? 2 : buf - 1;          // (s + 2) % 3
+        if (s + 2 < nsteps) fetch(s + 2, buf2);
+        const unsigned char* kb = lds_all + buf * kTileBytes;
         const int tok0 = s * kStep;
 
         if (QB == 1 || s < my_steps) {   // wavefronts whose queries end earlier skip the keys they cannot see
@@ -292,7 +313,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const u32x4 kf = *reinterpret_cast<const u32x4*>(kb + (16 * t + n) * kKRow + (32 * j + 8 * g) * 2);
+                const u32x4 kf = *reinterpret_cast<const u32x4*>(kb + 16 * t * kRowB + k_addr[j]);
 #pragma unroll
                 for (int u = 0; u < kNQ; ++u)
                     sc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf), qreg[u][j], sc[u][t], 0, 0, 0);
@@ -338,10 +359,9 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         // ---- O^T += V^T P^T, every V fragment used for both query tiles
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            // keys 8 g + n / 4 (lo) and 8 g + 4 + n / 4 (hi) sit in LDS rows 4 g + n / 4 and 16 + 4 g + n / 4
-            const unsigned char* src = vb + (4 * g + (n >> 2)) * kVRow + (16 * t + 4 * (n & 3)) * 2;
+            const unsigned char* src = kb + v_addr[t];
             const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src));
-            const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src + 16 * kVRow));
+            const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src + 16 * kRowB));
             const bf16x8 vt = __builtin_bit_cast(bf16x8, (i16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 #pragma unroll
             for (int u = 0; u < kNQ; ++u)
@@ -349,20 +369,11 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         }
         }
 
-        // Unconditional: after the last step this parks stale registers in a buffer nobody reads again,
-        // and in exchange every path through the loop has waited for this slot's loads, so the fetch
-        // into it at the top of the next step needs no wait that would also drain the newest loads.
-        stash(NEXT{}, (s + 1) & 1);
+        // tile s + 1 must be in LDS for everybody: own loads first, then the barrier
+        if (s + 2 < nsteps) landed_but_newest(); else landed_all();
         __syncthreads();
     };
-    {
-        int s = 0;
-        for (; s + 1 < nsteps; s += 2) {
-            step(S0{}, s);
-            step(S1{}, s + 1);
-        }
-        if (s < nsteps) step(S0{}, s);
-    }
+    for (int s = 0, buf = 0; s < nsteps; ++s, buf = buf == 2 ? 0 : buf + 1) step(s, buf);
 
     if (!live) return;
 #pragma unroll
@@ -387,7 +398,7 @@ int launch_tiled(const PrefillArgs& a, int64_t max_seqlen_q, int64_t num_seqs, i
     const int64_t q_per_wg = (int64_t)QB * kQBlock;
     const int parts = a.group / (WAVES / QB);
     dim3 grid((unsigned)((max_seqlen_q + q_per_wg - 1) / q_per_wg), (unsigned)num_seqs, (unsigned)(num_kv_heads * parts));
-    hipLaunchKernelGGL((paged_prefill_tile_kernel<WAVES, QB>), grid, dim3(64 * WAVES, 1, 1), 2 * kTileBytes, st, a);
+    hipLaunchKernelGGL((paged_prefill_tile_kernel<WAVES, QB>), grid, dim3(64 * WAVES, 1, 1), kRing * kTileBytes + kTblLds * 4, st, a);
     return (int)hipGetLastError();
 }
 

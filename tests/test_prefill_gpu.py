@@ -55,6 +55,16 @@ def test_block_sizes(gpu, bs):
     assert np.abs(f32(out) - oracle_paged(wl, kc, vc)).max() <= ATTN_ATOL
 
 
+@pytest.mark.parametrize("cached", [3008, 16512])
+def test_long_block_table_rows(gpu, cached):
+    """Sequences of 95 and 518 blocks (block size 32): the kernel keeps the first 512 block ids of a
+    sequence in LDS and looks the rest up in memory; tiles far into the ring's steady state."""
+    wl = workloads.make_prefill_workload("p", [cached + 40, 100], [cached, 0], 4, 2, bs=32, seed=cached,
+                                         pad_fraction=0.0).to(gpu)
+    out, kc, vc = run_paged(wl)
+    assert np.abs(f32(out) - oracle_paged(wl, kc, vc)).max() <= ATTN_ATOL
+
+
 def test_packed_keys_without_block_table_equals_causal_sdpa(gpu):
     """No prefix cached: K and V are the packed new rows and sq == sk, which reduces to
     scaled_dot_product_attention(is_causal=True), the convention of the reference's own attention
