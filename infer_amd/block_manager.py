@@ -90,6 +90,9 @@ class BlockManager:
         seq.block_table.clear()
 
     def can_append(self, seq: Sequence) -> bool:
+        # ``block_manager.py:120-121``: a free block is needed only by the first token of a new block
+        if len(seq) % self.block_size != 1:
+            return True
         return bool(self._lib.infer_pool_can_append(self._pool, len(seq)))
 
     def may_append(self, seq: Sequence):

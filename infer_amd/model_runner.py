@@ -144,6 +144,8 @@ class ModelRunner:
     def prepare_sample(self, seqs: list[Sequence]):
         temps = [seq.temperature for seq in seqs]
         all_greedy = all(t == 0 for t in temps)
+        if all_greedy:       # the sampler takes the argmax and never looks at the temperatures
+            return None, True
         t = torch.tensor(temps, dtype=torch.float32, pin_memory=True).to(self.device, non_blocking=True)
         return t, all_greedy
 
