@@ -191,11 +191,13 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     // step to arrive instead of two.  Here the waits are the explicit counts below.  M0 (the LDS base
     // of the transfer) is put back afterwards.
     typedef __attribute__((address_space(3))) void* lptr_t;
-    auto dma16 = [&](const uint16_t* src, unsigned char* dst) {
+    // Address = uniform 64-bit base (scalar registers) + per-lane 32-bit byte offset: no vector
+    // arithmetic per transfer.
+    auto dma16 = [&](const uint16_t* base, uint32_t byte_off, unsigned char* dst) {
         const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)dst;
         uint32_t keep;
-        __asm__ volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
-                         : "=&s"(keep) : "v"(src), "s"(lds_addr) : "memory");
+        __asm__ volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b32 m0, %0"
+                         : "=&s"(keep) : "v"(byte_off), "s"(base), "s"(lds_addr) : "memory");
     };
     constexpr int kLoads = (16 + WAVES - 1) / WAVES;
     const int tok_stride = (int)a.tok_stride;     // < 2^24 elements (checked on the host)
@@ -212,7 +214,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
         const int L = wave + i * WAVES < 16 ? wave + i * WAVES : 0;
-        ld_off[i] = (uint32_t)(ld_key(i) * tok_stride) + ld_col(i);
+        ld_off[i] = (uint32_t)(ld_key(i) * tok_stride) + ld_col(i);       // < 2^30: tok_stride < 2^24, 32 rows
         ld_dst[i] = (L >> 3) * kKTileBytes + (L & 7) * 1024;
     }
     // The first kTblLds block ids of the sequence are copied to LDS behind the ring (one barrier, before
@@ -252,8 +254,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         if (tok0 + kStep <= sk) {
 #pragma unroll
             for (int i = 0; i < kLoads; ++i) {
-                const uint16_t* src = (ld_dst[i] < kKTileBytes ? kp : vp) + ld_off[i];
-                dma16(src, dst + ld_dst[i]);
+                dma16(ld_dst[i] < kKTileBytes ? kp : vp, 2 * ld_off[i], dst + ld_dst[i]);
             }
         } else {
             // rows past the end of the sequence (last step only) re-read its last row: finite data whose
@@ -262,8 +263,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
             for (int i = 0; i < kLoads; ++i) {
                 const int r = ld_key(i) < last ? ld_key(i) : last;
-                const uint16_t* src = (ld_dst[i] < kKTileBytes ? kp : vp) + ((uint32_t)(r * tok_stride) + ld_col(i));
-                dma16(src, dst + ld_dst[i]);
+                dma16(ld_dst[i] < kKTileBytes ? kp : vp, 2 * ((uint32_t)(r * tok_stride) + ld_col(i)), dst + ld_dst[i]);
             }
         }
     };
