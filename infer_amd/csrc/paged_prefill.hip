@@ -80,22 +80,28 @@ __device__ __forceinline__ float max_xor32(float x) {
     return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
 }
 
-// LDS layout of a tile: key k of the step sits in row  16 ((k >> 2) & 1) + 4 (k >> 3) + (k & 3),  so
-// that the 16 K rows one ds_read_b128 pass touches (one MFMA row tile) and the 8 V rows one
-// transposing read pass touches are consecutive rows.  Rows are 256 B (no padding: the tiles are
-// written by global_load ... lds, which fills 1 KiB = four whole rows per wavefront instruction)
-// and the sixteen 16-byte chunks of row r are rotated by r positions (chunk c sits at position
-// (c + r) % 16), which spreads consecutive rows over the banks exactly like a 272-byte row stride
-// does (measured with a probe: plain 256 B rows cost 4x on both read patterns).
+// LDS layout of a tile.  Key k of the step is row  16 ((k >> 2) & 1) + 4 (k >> 3) + (k & 3)  of the
+// tile, so that the 16 K rows one ds_read_b128 pass touches (one MFMA row tile) and the 8 V rows one
+// transposing read pass touches are consecutive rows.  The tiles are written by
+// global_load ... lds, which fills 1 KiB (four rows) per wavefront instruction, lane l at byte 16 l;
+// which 16-byte chunk of which row a lane fetches is free, and the choice here interleaves the four
+// rows of such a group in pieces of 64 B (four chunks; four consecutive lanes still fetch 64
+// contiguous bytes of global memory): chunk c of row r sits at
+//     (r / 4) * 1040 + (c / 4) * 256 + (r % 4) * 64 + (c % 4) * 16
+// (groups are 1 KiB + 16 B apart).  The 16 rows of a K read then hit sixteen 16-byte slots that are all
+// different modulo 256, the 4 rows x 32 B of a transposing V read four 32-byte runs 64 B apart: no
+// bank is hit twice.  And the address of a read is one per-lane register plus a constant for every K
+// step, row tile and column tile, where a rotation of the chunks inside a row (the other
+// conflict-free choice for 256-byte rows) needs a register and an addition per read.
 constexpr int kNQ = 2;
 constexpr float kLazy = 8.f;
 constexpr int kQBlock = kNQ * kQTile;
-constexpr int kRowB = 256;
-constexpr int kKTileBytes = kStep * kRowB;
-constexpr int kVTileBytes = kStep * kRowB;
+constexpr int kGroupB = 1024 + 16;                        // four interleaved rows and the pad
+constexpr int kKTileBytes = (kStep / 4) * kGroupB;
+constexpr int kVTileBytes = (kStep / 4) * kGroupB;
 constexpr int kTileBytes = kKTileBytes + kVTileBytes;     // one K tile + one V tile
 constexpr int kRing = 3;                                  // tiles resident in LDS: consumed, landed, in flight
-constexpr int kTblLds = 512;                              // block ids of a sequence kept in LDS
+constexpr int kTblLds = 256;                              // block ids of a sequence kept in LDS
 __device__ __forceinline__ int tile_row(int k) { return 16 * ((k >> 2) & 1) + 4 * (k >> 3) + (k & 3); }
 __device__ __forceinline__ int tile_key(int r) { return (((r >> 2) & 3) << 3) | ((r >> 4) << 2) | (r & 3); }   // inverse of tile_row
 
@@ -203,19 +209,16 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     const int tok_stride = (int)a.tok_stride;     // < 2^24 elements (checked on the host)
     uint32_t ld_off[kLoads];                      // element offset inside a tile of what this lane fetches
     int ld_dst[kLoads];                           // LDS byte offset of the load inside a tile pair (uniform)
-    auto ld_key = [&](int i) {                    // key (row of the tile in memory) of load i of this lane
+    auto ld_key = [&](int i) {                    // key (row of the tile in memory) of load i of this lane:
         const int L = wave + i * WAVES < 16 ? wave + i * WAVES : 0;
-        return tile_key(4 * (L & 7) + (lane >> 4));
+        return tile_key(4 * (L & 7) + ((lane >> 2) & 3));              // lane l fills row (l / 4) % 4 of group L,
     };
-    auto ld_col = [&](int i) {                    // its element column
-        const int L = wave + i * WAVES < 16 ? wave + i * WAVES : 0;
-        return (uint32_t)(kvh * kD + (((lane & 15) - (4 * (L & 7) + (lane >> 4))) & 15) * 8);
-    };
+    auto ld_col = [&](int i) { return (uint32_t)(kvh * kD + ((lane & 3) + 4 * (lane >> 4)) * 8); };   // chunk l % 4 + 4 (l / 16)
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
         const int L = wave + i * WAVES < 16 ? wave + i * WAVES : 0;
         ld_off[i] = (uint32_t)(ld_key(i) * tok_stride) + ld_col(i);       // < 2^30: tok_stride < 2^24, 32 rows
-        ld_dst[i] = (L >> 3) * kKTileBytes + (L & 7) * 1024;
+        ld_dst[i] = (L >> 3) * kKTileBytes + (L & 7) * kGroupB;
     }
     // The first kTblLds block ids of the sequence are copied to LDS behind the ring (one barrier, before
     // anything is fetched): a lookup in memory, behind a division by the block size, would put some
@@ -271,18 +274,12 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     auto landed_but_newest = [&]() { __builtin_amdgcn_s_waitcnt(0x0F70 | kLoads); };
     auto landed_all = [&]() { __builtin_amdgcn_s_waitcnt(0x0F70); };
 
-    // Read addresses under the rotation.  K operand row n of MFMA row tile t is key
-    // 8 (n / 4) + 4 t + n % 4 = LDS row 16 t + n, K step j is chunk 4 j + g of it; V keys 8 g + n / 4 (lo)
-    // and 8 g + 4 + n / 4 (hi) sit in LDS rows 4 g + n / 4 and 16 more, columns 16 t + 4 (n % 4) .. + 3 are
-    // half n % 2 of chunk 2 t + (n % 4) / 2.  A row 16 further down has the same rotation.
-    int k_addr[4], v_addr[8];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) k_addr[j] = n * kRowB + (((4 * j + g + n) & 15) << 4);
-#pragma unroll
-    for (int t = 0; t < 8; ++t) {
-        const int row = 4 * g + (n >> 2);
-        v_addr[t] = kKTileBytes + row * kRowB + (((2 * t + ((n & 3) >> 1) + row) & 15) << 4) + (n & 1) * 8;
-    }
+    // Read addresses.  K operand row n of MFMA row tile t is key 8 (n / 4) + 4 t + n % 4 = tile row
+    // 16 t + n, K step j is chunk 4 j + g of it.  V keys 8 g + n / 4 (lo) and 8 g + 4 + n / 4 (hi) are
+    // tile rows 4 g + n / 4 and 16 more; columns 16 t + 4 (n % 4) .. + 3 are half n % 2 of chunk
+    // 2 t + (n % 4) / 2.
+    const int k_addr = (n >> 2) * kGroupB + (n & 3) * 64 + g * 16;
+    const int v_addr = kKTileBytes + g * kGroupB + (n >> 2) * 64 + ((n & 3) >> 1) * 16 + (n & 1) * 8;
 
     // tile s lives in ring buffer s % 3: requested at the top of step s - 2, landed (own loads counted,
     // then the barrier) at the end of step s - 1, read during step s; the buffer is requested again at
@@ -312,7 +309,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const u32x4 kf = *reinterpret_cast<const u32x4*>(kb + 16 * t * kRowB + k_addr[j]);
+                const u32x4 kf = *reinterpret_cast<const u32x4*>(kb + k_addr + 4 * t * kGroupB + j * 256);
 #pragma unroll
                 for (int u = 0; u < kNQ; ++u)
                     sc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf), qreg[u][j], sc[u][t], 0, 0, 0);
@@ -358,9 +355,9 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         // ---- O^T += V^T P^T, every V fragment used for both query tiles
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            const unsigned char* src = kb + v_addr[t];
+            const unsigned char* src = kb + v_addr + (t >> 1) * 256 + (t & 1) * 32;
             const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src));
-            const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src + 16 * kRowB));
+            const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src + 4 * kGroupB));
             const bf16x8 vt = __builtin_bit_cast(bf16x8, (i16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 #pragma unroll
             for (int u = 0; u < kNQ; ++u)
