@@ -65,6 +65,27 @@ def test_long_block_table_rows(gpu, cached):
     assert np.abs(f32(out) - oracle_paged(wl, kc, vc)).max() <= ATTN_ATOL
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_random_ragged_batches(gpu, seed):
+    """Random head shapes, block sizes, lengths and cached prefixes (prefix lengths are whole blocks, as
+    the block manager hands them out): every path of the tile ring (first, steady, last partial tile,
+    several query blocks per workgroup) against the oracle."""
+    rng = np.random.default_rng(1000 + seed)
+    hkv = int(rng.choice([1, 2, 4, 8]))
+    hq = hkv * int(rng.choice([1, 2, 3, 4, 6, 8]))
+    bs = int(rng.choice([32, 64, 256]))
+    nseq = int(rng.integers(1, 7))
+    lens, cached = [], []
+    for _ in range(nseq):
+        c = int(rng.integers(0, 4)) * bs if rng.random() < 0.5 else 0
+        n = c + int(rng.integers(1, 400))
+        lens.append(n); cached.append(c)
+    wl = workloads.make_prefill_workload("r", lens, cached, hq, hkv, bs=bs, seed=seed, pad_fraction=0.05).to(gpu)
+    out, kc, vc = run_paged(wl)
+    err = np.abs(f32(out) - oracle_paged(wl, kc, vc)).max()
+    assert err <= ATTN_ATOL, (hq, hkv, bs, lens, cached, float(err))
+
+
 def test_packed_keys_without_block_table_equals_causal_sdpa(gpu):
     """No prefix cached: K and V are the packed new rows and sq == sk, which reduces to
     scaled_dot_product_attention(is_causal=True), the convention of the reference's own attention
