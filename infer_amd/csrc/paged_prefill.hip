@@ -12,9 +12,9 @@
 //   S^T[key, query] = K[key, :] . Q^T       2 row tiles x 4 v_mfma_f32_16x16x32_bf16 per column tile
 //   online softmax in the accumulator layout (lane = query, 8 keys per lane)
 //   O^T[d, query]  += V^T[d, key] . P^T     8 MFMAs per column tile
-// A workgroup is 4 to 8 wavefronts that read the same keys: the query heads of one KV head (all of
-// them, or a divisor-sized part when the group is larger than 8) times as many consecutive query
-// blocks as fit (4 blocks for a group of 1, 2 for groups of 2 and 3, 1 otherwise).  They share
+// A workgroup is 3 or 4 wavefronts that read the same keys: up to four query heads of one KV head
+// (the largest divisor of the group size that is at most 4) times as many consecutive query blocks
+// as fit (4 blocks for one head, 2 for two, 1 otherwise).  They share
 // every 32-key K tile and V tile through LDS: the tiles are fetched once per workgroup, straight
 // from global memory into a ring of three LDS buffers (global_load_dwordx4 ... lds: no registers, no
 // LDS store instructions; tile s + 2 is in flight while tile s + 1 has landed and tile s is consumed;
@@ -420,11 +420,16 @@ extern "C" int infer_paged_prefill_bf16(const void* q, int64_t q_stride0, const 
     if (num_seqs > 65535 || num_kv_heads * 16 > 65535) return INFER_KV_EINVAL;
     if (kv_token_stride > (1 << 24)) return INFER_KV_EUNSUPPORTED;   // 32-bit offsets inside a tile
     const int G = (int)(num_q_heads / num_kv_heads);
-    // Workgroup shape: the heads of the group (or its largest divisor up to 8) times the number of
-    // consecutive query blocks that brings the workgroup to 4 - 8 wavefronts.
+    // Workgroup shape: the largest divisor of the group size up to 4 as query heads, times the number
+    // of consecutive query blocks that brings the workgroup to 3 - 4 wavefronts.  Small workgroups
+    // win: three or four of them share a compute unit, each with its own barrier, where one workgroup
+    // of 6 - 8 wavefronts (all heads of a large group) keeps every wavefront of the unit in lockstep
+    // (measured on 8 x 2048-token prompts, TFLOP/s: G = 8 as 8 heads 526, as 2 x 4 heads 629; G = 6 as
+    // 6 heads 408, as 2 x 3 heads 528; G = 5 as 5 heads 340, as 5 x 1 head with 4 query blocks 507).
     int heads = 1;
-    for (int h = G < 8 ? G : 8; h >= 1; --h)
+    for (int h = G < 4 ? G : 4; h >= 1; --h)
         if (G % h == 0) { heads = h; break; }
+    const int qb = heads == 1 ? 4 : (heads == 2 ? 2 : 1);
     PrefillArgs a;
     a.q = (const uint16_t*)q; a.q_stride0 = q_stride0;
     a.k = (const uint16_t*)k; a.v = (const uint16_t*)v;
@@ -432,20 +437,17 @@ extern "C" int infer_paged_prefill_bf16(const void* q, int64_t q_stride0, const 
     a.out = (uint16_t*)out; a.out_stride0 = out_stride0;
     a.cu_q = cu_seqlens_q; a.cu_k = cu_seqlens_k;
     a.bt = block_table; a.bt_stride0 = bt_stride0;
-    a.group = G; a.heads_per_wg = heads; a.qblocks_per_wg = heads == 1 ? 4 : (heads <= 3 ? 2 : 1);
+    a.group = G;
     a.block_size = (int)block_size; a.num_blocks = (int)num_blocks;
     a.scale_log2 = scale * 1.4426950408889634f;
     a.causal = causal ? 1 : 0;
     hipStream_t st = (hipStream_t)stream;
+    a.heads_per_wg = heads; a.qblocks_per_wg = qb;
     switch (heads) {
         case 1: return launch_tiled<4, 4>(a, max_seqlen_q, num_seqs, num_kv_heads, st);
         case 2: return launch_tiled<4, 2>(a, max_seqlen_q, num_seqs, num_kv_heads, st);
-        case 3: return launch_tiled<6, 2>(a, max_seqlen_q, num_seqs, num_kv_heads, st);
+        case 3: return launch_tiled<3, 1>(a, max_seqlen_q, num_seqs, num_kv_heads, st);
         case 4: return launch_tiled<4, 1>(a, max_seqlen_q, num_seqs, num_kv_heads, st);
-        case 5: return launch_tiled<5, 1>(a, max_seqlen_q, num_seqs, num_kv_heads, st);
-        case 6: return launch_tiled<6, 1>(a, max_seqlen_q, num_seqs, num_kv_heads, st);
-        case 7: return launch_tiled<7, 1>(a, max_seqlen_q, num_seqs, num_kv_heads, st);
-        case 8: return launch_tiled<8, 1>(a, max_seqlen_q, num_seqs, num_kv_heads, st);
         default: return INFER_KV_EUNSUPPORTED;
     }
 }
