@@ -93,6 +93,7 @@ class ModelRunner:
         host = self.stage_host.numpy()
         self.h_input_ids, self.h_seq_lens = host[:n], host[n:2 * n]
         self.h_block_tables = host[2 * n:].reshape(n, m)
+        self._staged_tables = [None] * n        # what each host row of the block table currently holds
         self.d_input_ids, self.d_seq_lens = self.stage_dev[:n], self.stage_dev[n:2 * n]
         self.d_block_tables = self.stage_dev[2 * n:].view(n, m)
         self.d_positions = torch.zeros(n, dtype=torch.int64, device=self.device)
@@ -117,13 +118,17 @@ class ModelRunner:
             raise RuntimeError(f"decode batch of {bs} exceeds max_num_seqs={self.max_bs}")
         run_bs = bs if self.enforce_eager or not self.graph_bs else next(x for x in self.graph_bs if x >= bs)
         ids, lens, tables = self.h_input_ids, self.h_seq_lens, self.h_block_tables
+        ids[:bs] = [seq.last_token for seq in seqs]
+        lens[:bs] = [len(seq) for seq in seqs]
+        staged = self._staged_tables
         for i, seq in enumerate(seqs):
-            ids[i] = seq.last_token
-            lens[i] = len(seq)
-            bt = seq.block_table
+            bt = tuple(seq.block_table)
+            if staged[i] == bt:          # a row changes once per block of tokens: skip the rewrite otherwise
+                continue
             if len(bt) > self.max_num_blocks:
                 raise RuntimeError(f"sequence of {len(seq)} tokens exceeds max_model_len={self.config.max_model_len}")
             tables[i, :len(bt)] = bt
+            staged[i] = bt
         ids[bs:run_bs] = 0
         lens[bs:run_bs] = 0           # padding rows: no append, no attention
         self.stage_dev.copy_(self.stage_host, non_blocking=True)
