@@ -78,19 +78,33 @@ __device__ __forceinline__ u32x4 load16(const uint16_t* p) {
 
 __device__ __forceinline__ int steps_of(int len) { return len > 0 ? (len + kStep - 1) / kStep : 0; }
 
-__device__ __forceinline__ int wave_sum(int x) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
+// Inclusive prefix sum over the 64 lanes on the vector pipe (data-parallel primitives): shifts by 1,
+// 2, 4 and 8 inside each row of 16 lanes, then the last lane of row 0 (2) is added to row 1 (3) and the
+// last lane of the lower half to the upper half.  Six instructions, where shuffles would be six round
+// trips through LDS in front of the first load of the kernel.
+__device__ __forceinline__ int wave_inclusive_scan(int x, int) {
+    x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xf, 0xf, false);   // row_shr:1
+    x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xf, 0xf, false);   // row_shr:2
+    x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xf, 0xf, false);   // row_shr:4
+    x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xf, 0xf, false);   // row_shr:8
+    x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xa, 0xf, false);   // row_bcast:15 into rows 1 and 3
+    x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xc, 0xf, false);   // row_bcast:31 into rows 2 and 3
     return x;
 }
 
-__device__ __forceinline__ int wave_inclusive_scan(int x, int lane) {
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        int y = __shfl_up(x, o);
-        if (lane >= o) x += y;
-    }
-    return x;
+__device__ __forceinline__ int wave_sum(int x) { return __builtin_amdgcn_readlane(wave_inclusive_scan(x, 0), 63); }
+
+// Minimum over the 64 lanes, the same ladder with min in place of +.
+__device__ __forceinline__ int wave_min(int x) {
+    auto step = [](int v, int moved) { return moved < v ? moved : v; };
+    const int top = 0x7fffffff;
+    x = step(x, __builtin_amdgcn_update_dpp(top, x, 0x111, 0xf, 0xf, false));
+    x = step(x, __builtin_amdgcn_update_dpp(top, x, 0x112, 0xf, 0xf, false));
+    x = step(x, __builtin_amdgcn_update_dpp(top, x, 0x114, 0xf, 0xf, false));
+    x = step(x, __builtin_amdgcn_update_dpp(top, x, 0x118, 0xf, 0xf, false));
+    x = step(x, __builtin_amdgcn_update_dpp(top, x, 0x142, 0xa, 0xf, false));
+    x = step(x, __builtin_amdgcn_update_dpp(top, x, 0x143, 0xc, 0xf, false));
+    return __builtin_amdgcn_readlane(x, 63);
 }
 
 // max over lanes l and l ^ 16 (l ^ 32) in every lane.  v_permlane16_swap exchanges the odd 16-lane rows
@@ -456,12 +470,7 @@ __global__ void __launch_bounds__(512) paged_decode_split_kernel(DecodeArgs a) {
         const bool ok = lane < W / 4;
         const int share = ok ? (total + cand - 1) / cand : 0;
         int key = ok ? ((share * cand - total) << 7) | lane : 0x7fffffff;   // lane < 64 < 128
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            const int other = __shfl_xor(key, o);
-            key = other < key ? other : key;
-        }
-        spans = W - (__builtin_amdgcn_readfirstlane(key) & 127);
+        spans = W - (wave_min(key) & 127);
     }
     if (w == 0 && h == 0 && lane == 0) {
         a.header[0] = spans;
