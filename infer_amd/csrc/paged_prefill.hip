@@ -194,19 +194,23 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     // The load is issued as inline assembly on purpose.  Through the compiler's builtin every later
     // LDS read is preceded by a wait for ALL outstanding loads (the compiler cannot see that a read
     // touches another ring buffer than the one being filled), which would leave the newest tile half a
-    // step to arrive instead of two.  Here the waits are the explicit counts below.  M0 (the LDS base
-    // of the transfer) is put back afterwards.
-    typedef __attribute__((address_space(3))) void* lptr_t;
+    // step to arrive instead of two.  Here the waits are the explicit counts below.  M0 holds the LDS
+    // base of the transfer; nothing else in this kernel uses M0 (no other LDS transfer, no indexed
+    // register access), so it is not saved: the scalar instructions of a transfer are on the critical
+    // path of every step.
     // Address = uniform 64-bit base (scalar registers) + per-lane 32-bit byte offset: no vector
     // arithmetic per transfer.
+    typedef __attribute__((address_space(3))) void* lptr_t;
     auto dma16 = [&](const uint16_t* base, uint32_t byte_off, unsigned char* dst) {
         const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)dst;
-        uint32_t keep;
-        __asm__ volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b32 m0, %0"
-                         : "=&s"(keep) : "v"(byte_off), "s"(base), "s"(lds_addr) : "memory");
+        __asm__ volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                         :: "v"(byte_off), "s"(base), "s"(lds_addr) : "memory");
     };
     constexpr int kLoads = (16 + WAVES - 1) / WAVES;
     const int tok_stride = (int)a.tok_stride;     // < 2^24 elements (checked on the host)
+    // loads 0 .. 7 are the K tile, 8 .. 15 the V tile: with four wavefronts (load w + 4 i) that is a
+    // matter of i alone
+    auto load_is_k = [&](int i) { return WAVES == 4 ? i < 2 : (wave + i * WAVES < 16 ? wave + i * WAVES : 0) < 8; };
     uint32_t ld_off[kLoads];                      // element offset inside a tile of what this lane fetches
     int ld_dst[kLoads];                           // LDS byte offset of the load inside a tile pair (uniform)
     auto ld_key = [&](int i) {                    // key (row of the tile in memory) of load i of this lane:
@@ -257,7 +261,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         if (tok0 + kStep <= sk) {
 #pragma unroll
             for (int i = 0; i < kLoads; ++i) {
-                dma16(ld_dst[i] < kKTileBytes ? kp : vp, 2 * ld_off[i], dst + ld_dst[i]);
+                dma16(load_is_k(i) ? kp : vp, 2 * ld_off[i], dst + ld_dst[i]);
             }
         } else {
             // rows past the end of the sequence (last step only) re-read its last row: finite data whose
@@ -266,7 +270,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
             for (int i = 0; i < kLoads; ++i) {
                 const int r = ld_key(i) < last ? ld_key(i) : last;
-                dma16(ld_dst[i] < kKTileBytes ? kp : vp, 2 * ((uint32_t)(r * tok_stride) + ld_col(i)), dst + ld_dst[i]);
+                dma16(load_is_k(i) ? kp : vp, 2 * ((uint32_t)(r * tok_stride) + ld_col(i)), dst + ld_dst[i]);
             }
         }
     };
