@@ -332,9 +332,12 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
                 for (int e = 0; e < 4; ++e) sv[4 * t + e] = sc[u][t][e];
             if (tok0 + kStep - 1 > lim_lo[u]) {      // wave-uniform: off the diagonal no lane masks anything
+                // key tok0 + 8 g + i is masked iff i > rel; written so that nothing but this one
+                // subtraction could be computed ahead of the branch
+                const int rel = my_limit[u] - tok0 - 8 * g;
 #pragma unroll
                 for (int i = 0; i < 8; ++i)
-                    if (tok0 + 8 * g + i > my_limit[u]) sv[i] = -INFINITY;
+                    if (i > rel) sv[i] = -INFINITY;
             }
             float mx = sv[0];
 #pragma unroll
