@@ -170,9 +170,17 @@ def main():
                     it[0] += 1
                     _lib.check(lib.infer_kv_probe_copy(bufs[i].data_ptr(), dst.data_ptr(), nbytes, wg, stream), "probe")
                 return f
+            def rds(wg):
+                def f():
+                    i = it[0] % 4
+                    it[0] += 1
+                    _lib.check(lib.infer_kv_probe_read_streaming(bufs[i].data_ptr(), nbytes, sink.data_ptr(), wg, stream), "probe")
+                return f
             for wg in (256, 512, 1024):
                 ms = gpu_time_ms(rd(wg), 30, 3)
                 res[f"read_{label}_{wg}wg_GBps"] = round(nbytes / ms / 1e6, 1)
+                ms = gpu_time_ms(rds(wg), 30, 3)
+                res[f"read_streaming_hint_{label}_{wg}wg_GBps"] = round(nbytes / ms / 1e6, 1)
             for wg in (2048, 8192):
                 ms = gpu_time_ms(cp(wg), 30, 3)
                 res[f"copy_{label}_{wg}wg_GBps_read_plus_write"] = round(2 * nbytes / ms / 1e6, 1)

@@ -44,6 +44,7 @@ SIGNATURES = {
     "infer_rms_norm_splitk_bf16": (_c.c_int, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _f32,
                                               _vp]),
     "infer_kv_probe_read": (_c.c_int, [_vp, _sz, _vp, _c.c_int, _vp]),
+    "infer_kv_probe_read_streaming": (_c.c_int, [_vp, _sz, _vp, _c.c_int, _vp]),
     "infer_kv_probe_copy": (_c.c_int, [_vp, _vp, _sz, _c.c_int, _vp]),
     "infer_pool_create": (_vp, [_i32, _i32]),
     "infer_pool_destroy": (None, [_vp]),

@@ -13,7 +13,12 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ uint32_t fold(u32x4 a) { return a.x ^ a.y ^ a.z ^ a.w; }
 
-// Each workgroup reads a contiguous share of the buffer exactly once.
+// Each workgroup reads a contiguous share of the buffer exactly once.  STREAM: with the streaming
+// (nontemporal) hint the decode kernel puts on its K and V loads.
+template <bool STREAM>
+__device__ __forceinline__ u32x4 probe_load(const u32x4* p) { return STREAM ? __builtin_nontemporal_load(p) : *p; }
+
+template <bool STREAM>
 __global__ void __launch_bounds__(512) stream_read_kernel(const u32x4* __restrict__ src, size_t n_vec, uint32_t* sink) {
     const size_t per = n_vec / gridDim.x;
     const u32x4* p = src + per * blockIdx.x;
@@ -22,11 +27,11 @@ __global__ void __launch_bounds__(512) stream_read_kernel(const u32x4* __restric
     for (; i + 7 * 512 < per; i += 8 * 512) {
         u32x4 r[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) r[u] = p[i + u * 512];
+        for (int u = 0; u < 8; ++u) r[u] = probe_load<STREAM>(p + i + u * 512);
 #pragma unroll
         for (int u = 0; u < 8; ++u) acc ^= fold(r[u]);
     }
-    for (; i < per; i += 512) acc ^= fold(p[i]);
+    for (; i < per; i += 512) acc ^= fold(probe_load<STREAM>(p + i));
     if (acc == 0x9e3779b9u) *sink = acc;   // keeps the loads alive; practically never true
 }
 
@@ -49,7 +54,14 @@ extern "C" {
 
 int infer_kv_probe_read(const void* src, size_t bytes, void* sink4, int workgroups, void* stream) {
     if (!src || !sink4 || bytes < 16 || workgroups <= 0 || ((uintptr_t)src & 15)) return INFER_KV_EINVAL;
-    hipLaunchKernelGGL(stream_read_kernel, dim3(workgroups), dim3(512), 0, (hipStream_t)stream, (const u32x4*)src,
+    hipLaunchKernelGGL(stream_read_kernel<false>, dim3(workgroups), dim3(512), 0, (hipStream_t)stream, (const u32x4*)src,
+                       bytes / 16, (uint32_t*)sink4);
+    return (int)hipGetLastError();
+}
+
+int infer_kv_probe_read_streaming(const void* src, size_t bytes, void* sink4, int workgroups, void* stream) {
+    if (!src || !sink4 || bytes < 16 || workgroups <= 0 || ((uintptr_t)src & 15)) return INFER_KV_EINVAL;
+    hipLaunchKernelGGL(stream_read_kernel<true>, dim3(workgroups), dim3(512), 0, (hipStream_t)stream, (const u32x4*)src,
                        bytes / 16, (uint32_t*)sink4);
     return (int)hipGetLastError();
 }
