@@ -99,19 +99,6 @@ __device__ __forceinline__ int wave_inclusive_scan(int x, int) {
 
 __device__ __forceinline__ int wave_sum(int x) { return __builtin_amdgcn_readlane(wave_inclusive_scan(x, 0), 63); }
 
-// Minimum over the 64 lanes, the same ladder with min in place of +.
-__device__ __forceinline__ int wave_min(int x) {
-    auto step = [](int v, int moved) { return moved < v ? moved : v; };
-    const int top = 0x7fffffff;
-    x = step(x, __builtin_amdgcn_update_dpp(top, x, 0x111, 0xf, 0xf, false));
-    x = step(x, __builtin_amdgcn_update_dpp(top, x, 0x112, 0xf, 0xf, false));
-    x = step(x, __builtin_amdgcn_update_dpp(top, x, 0x114, 0xf, 0xf, false));
-    x = step(x, __builtin_amdgcn_update_dpp(top, x, 0x118, 0xf, 0xf, false));
-    x = step(x, __builtin_amdgcn_update_dpp(top, x, 0x142, 0xa, 0xf, false));
-    x = step(x, __builtin_amdgcn_update_dpp(top, x, 0x143, 0xc, 0xf, false));
-    return __builtin_amdgcn_readlane(x, 63);
-}
-
 // max over lanes l and l ^ 16 (l ^ 32) in every lane.  v_permlane16_swap exchanges the odd 16-lane rows
 // of its first operand with the even rows of its second: fed the same value twice it returns
 // (rows 0 0 2 2, rows 1 1 3 3), whose maximum is the reduction; v_permlane32_swap does the same with
@@ -463,19 +450,16 @@ __global__ void __launch_bounds__(512) paged_decode_split_kernel(DecodeArgs a) {
     // every step gets a workgroup of its own: on tiny problems a longer span would only serialise
     // memory latency (measured: one sequence of 512 tokens 14.7 -> 6.7 us).
     //
-    // The share is a whole number of steps, so with `rem` left over most workgroups idle for the
-    // last step of the launch (64 sequences of about 2450 tokens: 4906 steps over 256 workgroups = 19 each and 42 with 20, i.e.
-    // 214 compute units wait out a twentieth of the run).  Each lane therefore tries one span
-    // count in (3W/4, W] and the wave keeps the one whose rounded-up shares waste the fewest steps
-    // (ties: the larger count); the workgroups beyond it leave at once.  Bandwidth is flat over
-    // that range of resident workgroups, so the shorter tail is a pure gain.
+    // A launch takes as long as its longest span (a sweep over forced span counts on 4907 steps:
+    // 102-103 us at 20 steps per workgroup, 104-105 at 22, 108 at 23-24, 113 at 26), so the longest
+    // span is made as short as the grid allows, ceil(total / W) steps, and then the fewest workgroups
+    // that reach it are used: the shares are as even as whole steps permit (4907 steps, 256
+    // workgroups: 246 spans of 19 or 20 steps instead of 42 of 20 and 214 of 19); the workgroups beyond
+    // the span count leave at once.
     int spans = W;
-    if (total > W && W >= 4) {
-        const int cand = W - lane;
-        const bool ok = lane < W / 4;
-        const int share = ok ? (total + cand - 1) / cand : 0;
-        int key = ok ? ((share * cand - total) << 7) | lane : 0x7fffffff;   // lane < 64 < 128
-        spans = W - (wave_min(key) & 127);
+    if (total > W) {
+        const int longest = (total + W - 1) / W;
+        spans = (total + longest - 1) / longest;
     }
     if (w == 0 && h == 0 && lane == 0) {
         a.header[0] = spans;
