@@ -744,6 +744,8 @@ int infer_paged_decode_merge_bf16(void* out, int64_t out_stride0, const int32_t*
     if (head_dim != kD) return INFER_KV_EUNSUPPORTED;
     if (num_q_heads % num_kv_heads != 0 || num_q_heads / num_kv_heads > 16) return INFER_KV_EUNSUPPORTED;
     if (out_stride0 < num_q_heads * kD) return INFER_KV_EINVAL;
+    // 8-byte stores of four outputs; 16-byte loads of the records
+    if (((uintptr_t)out & 7) || (out_stride0 & 3) || ((uintptr_t)workspace & 15)) return INFER_KV_EALIGN;
     const int G = (int)(num_q_heads / num_kv_heads);
     DecodeWorkspace ws = decode_workspace_layout(batch, G, num_kv_heads);
     if (ws.total_bytes > workspace_bytes) return INFER_KV_EWORKSPACE;
@@ -773,7 +775,9 @@ int infer_paged_decode_bf16(const void* q, int64_t q_stride0, const void* k_cach
                             const int32_t* context_lens, int64_t batch, int64_t num_q_heads,
                             int64_t num_kv_heads, int64_t head_dim, int64_t block_size, int64_t num_blocks,
                             float scale, void* workspace, size_t workspace_bytes, void* stream) {
-    if (!out) return INFER_KV_EINVAL;
+    // what the merge launch would reject is rejected before the split launch is enqueued
+    if (!out || out_stride0 < num_q_heads * kD) return INFER_KV_EINVAL;
+    if (((uintptr_t)out & 7) || (out_stride0 & 3)) return INFER_KV_EALIGN;
     int rc = infer_paged_decode_split_bf16(q, q_stride0, k_cache, v_cache, cache_block_stride, cache_token_stride,
                                            block_table, bt_stride0, context_lens, batch, num_q_heads,
                                            num_kv_heads, head_dim, block_size, num_blocks, scale, workspace,

@@ -58,5 +58,11 @@ def test_argument_errors_are_reported_before_anything_is_launched():
     assert lib.infer_kv_append_bf16(p16 + 2, 1024, p16, 1024, p16, p16, p16, 4, 1024, 256, None) == -2
     assert lib.infer_paged_decode_bf16(None, 0, None, None, 0, 0, None, 0, None, 0, None,
                                        1, 32, 8, 128, 256, 4, 1.0, None, 0, None) == -1
+    # the combined decode call rejects what its second launch would reject before the first is enqueued
+    assert lib.infer_paged_decode_bf16(p16, 4096, p16, p16, 262144, 1024, p16 + 2, 4096, p16, 1, p16,
+                                       1, 32, 8, 128, 256, 4, 1.0, p16, 1 << 30, None) == -2    # out not 8-byte aligned
+    assert lib.infer_paged_decode_bf16(p16, 4096, p16, p16, 262144, 1024, p16, 4095, p16, 1, p16,
+                                       1, 32, 8, 128, 256, 4, 1.0, p16, 1 << 30, None) == -1    # out rows overlap
+    assert lib.infer_paged_decode_merge_bf16(p16 + 4, 4096, p16, 1, 32, 8, 128, p16, 1 << 30, None) == -2
     with pytest.raises(RuntimeError, match="workspace too small"):
         _lib.check(-3, "x")
