@@ -152,9 +152,9 @@ def main():
         stream = torch.cuda.current_stream().cuda_stream
         sink = torch.zeros(4, dtype=torch.uint8, device=dev)
         res = {"ceiling_run": True, "method": "HIP events, 30 launches after 3 warm-ups, buffers rotated (4 x size)"}
-        for label, nbytes in (("640MB", 640 * 10 ** 6 // 16 * 16), ("2GiB", 1 << 31)):
+        for label, nbytes in (("54MB", 13184 * 4096), ("640MB", 640 * 10 ** 6 // 4096 * 4096), ("2GiB", 1 << 31)):
             bufs = [torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(4)]
-            dst = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            dsts = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(2)]
             it = [0]
 
             def rd(wg):
@@ -176,6 +176,16 @@ def main():
                     it[0] += 1
                     _lib.check(lib.infer_kv_probe_read_streaming(bufs[i].data_ptr(), nbytes, sink.data_ptr(), wg, stream), "probe")
                 return f
+            def cprows():
+                i = it[0] % 4
+                it[0] += 1
+                _lib.check(lib.infer_kv_probe_copy_rows(bufs[i].data_ptr(), dsts[i % 2].data_ptr(), nbytes, stream), "probe")
+            ms = gpu_time_ms(cprows, 32, 4)
+            res[f"copy_one_wave_per_4KiB_{label}_GBps_read_plus_write"] = round(2 * nbytes / ms / 1e6, 1)
+            if label == "54MB":    # the size of one prefill step's append; the other probes are for the large sizes
+                del bufs, dsts
+                continue
+            dst = dsts[0]
             for wg in (256, 512, 1024):
                 ms = gpu_time_ms(rd(wg), 30, 3)
                 res[f"read_{label}_{wg}wg_GBps"] = round(nbytes / ms / 1e6, 1)
@@ -184,7 +194,7 @@ def main():
             for wg in (2048, 8192):
                 ms = gpu_time_ms(cp(wg), 30, 3)
                 res[f"copy_{label}_{wg}wg_GBps_read_plus_write"] = round(2 * nbytes / ms / 1e6, 1)
-            del bufs, dst
+            del bufs, dst, dsts
         print(json.dumps(res))
         return
     if args.append_sweep:
@@ -211,6 +221,30 @@ def main():
             res[f"rows_{n}"] = {"us": round(ms * 1e3, 2), "GBps": round(nbytes / ms / 1e6, 1),
                                 "frac_of_8TBps": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
             del srcs, slots
+        # the same kernel on three slot layouts (the sweep above is the fully scattered one)
+        for n in (13824, 65536):
+            reps = max(2, min(16, (600 << 20) // (n * 4 * dkv)))
+            srcs = [(torch.randn((n, 8, 128), dtype=torch.bfloat16, device=dev),
+                     torch.randn((n, 8, 128), dtype=torch.bfloat16, device=dev)) for _ in range(reps)]
+
+            def whole_blocks():
+                blk = torch.randperm(pool_rows // 256, device=dev)[:n // 256]
+                return (blk[:, None] * 256 + torch.arange(256, device=dev)[None, :]).reshape(-1).to(torch.int32)
+            layouts = {"sequential": [torch.arange(n, device=dev, dtype=torch.int32)] * reps,
+                       "whole_blocks_shuffled": [whole_blocks() for _ in range(reps)],
+                       "rows_scattered": [torch.randperm(pool_rows, device=dev)[:n].to(torch.int32) for _ in range(reps)]}
+            for name, slots in layouts.items():
+                it = [0]
+
+                def step_layout():
+                    i = it[0]
+                    it[0] += 1
+                    kc, vc = caches[i % 2]
+                    ops.store_kvcache(srcs[i % reps][0], srcs[i % reps][1], kc, vc, slots[i % reps])
+                ms = gpu_time_ms(step_layout, 100, 10)
+                nbytes = workloads.append_algorithmic_bytes(n, n, dkv)
+                res[f"layout_{name}_{n}"] = {"us": round(ms * 1e3, 2), "GBps": round(nbytes / ms / 1e6, 1)}
+            del srcs, layouts
         print(json.dumps(res))
         return
     if args.splits:

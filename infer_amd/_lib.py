@@ -46,6 +46,7 @@ SIGNATURES = {
     "infer_kv_probe_read": (_c.c_int, [_vp, _sz, _vp, _c.c_int, _vp]),
     "infer_kv_probe_read_streaming": (_c.c_int, [_vp, _sz, _vp, _c.c_int, _vp]),
     "infer_kv_probe_copy": (_c.c_int, [_vp, _vp, _sz, _c.c_int, _vp]),
+    "infer_kv_probe_copy_rows": (_c.c_int, [_vp, _vp, _sz, _vp]),
     "infer_pool_create": (_vp, [_i32, _i32]),
     "infer_pool_destroy": (None, [_vp]),
     "infer_pool_last_error": (_c.c_char_p, []),

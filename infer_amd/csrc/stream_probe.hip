@@ -2,6 +2,7 @@
 // with the same launch shape as the decode kernel (one workgroup of 512 threads per span, 16-byte
 // loads, three batches of eight loads in flight per lane).  Not part of the KV-cache path; bench.py
 // --ceiling uses it to put the kernels' achieved bandwidth next to the practical ceiling of the part.
+// Two copy shapes: a grid-stride loop, and the append kernel's own shape (one wavefront per 4 KiB).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -48,6 +49,21 @@ __global__ void __launch_bounds__(256) stream_copy_kernel(const u32x4* __restric
     for (; i < n_vec; i += stride) dst[i] = src[i];
 }
 
+// The append kernel's launch shape on contiguous memory: one wavefront copies 4 KiB (a K row and a
+// V row of 2 KiB), four loads then four stores per lane, no loop; 256-thread workgroups.
+__global__ void __launch_bounds__(256) stream_copy_rows_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst,
+                                                               size_t n_vec) {
+    const size_t wave = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 6;
+    const int lane = threadIdx.x & 63;
+    const size_t base = wave * 256;
+    if (base + 256 > n_vec) return;
+    u32x4 r[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) r[u] = __builtin_nontemporal_load(src + base + lane + 64 * u);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) __builtin_nontemporal_store(r[u], dst + base + lane + 64 * u);
+}
+
 }  // namespace
 
 extern "C" {
@@ -70,6 +86,15 @@ int infer_kv_probe_copy(const void* src, void* dst, size_t bytes, int workgroups
     if (!src || !dst || bytes < 16 || workgroups <= 0 || (((uintptr_t)src | (uintptr_t)dst) & 15)) return INFER_KV_EINVAL;
     hipLaunchKernelGGL(stream_copy_kernel, dim3(workgroups), dim3(256), 0, (hipStream_t)stream, (const u32x4*)src,
                        (u32x4*)dst, bytes / 16);
+    return (int)hipGetLastError();
+}
+
+int infer_kv_probe_copy_rows(const void* src, void* dst, size_t bytes, void* stream) {
+    if (!src || !dst || bytes < 4096 || (((uintptr_t)src | (uintptr_t)dst) & 15)) return INFER_KV_EINVAL;
+    const size_t rows = bytes / 4096;           // a tail shorter than 4 KiB is not copied
+    if ((rows + 3) / 4 > 0x7fffffffULL) return INFER_KV_EINVAL;
+    hipLaunchKernelGGL(stream_copy_rows_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, (hipStream_t)stream,
+                       (const u32x4*)src, (u32x4*)dst, rows * 256);
     return (int)hipGetLastError();
 }
 
