@@ -91,16 +91,23 @@ __global__ void __launch_bounds__(256) skinny_gemm_kernel(GemmArgs a) {
 
     auto issue_w = [&](auto SLOT, int c) {
         constexpr int slot = decltype(SLOT)::value;
-        const int64_t off = (int64_t)(c < a.chunks ? c : a.chunks - 1) * kKC;
+        // Past the end of the slice every lane requests the same few bytes at the start of the matrix
+        // instead (a request that is never used but keeps the count of loads in flight the same on
+        // every step, so the waits stay exact): re-reading the last chunk would add 2 chunks of
+        // traffic to a slice of 4 to 12.
+        const bool live = c < a.chunks;
+        const int64_t off = (int64_t)c * kKC;
 #pragma unroll
-        for (int r = 0; r < kR; ++r)
+        for (int r = 0; r < kR; ++r) {
+            const uint16_t* p = live ? wp[r] + off : a.w;
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk) wreg[slot][r][kk] = load16_stream(wp[r] + off + 32 * kk);
+            for (int kk = 0; kk < 4; ++kk) wreg[slot][r][kk] = load16_stream(p + 32 * kk);
+        }
     };
     auto issue_x = [&](int c) {
-        const int cc = c < a.chunks ? c : a.chunks - 1;
+        const bool live = c < a.chunks;
 #pragma unroll
-        for (int i = 0; i < MT; ++i) xreg[i] = load16(xp[i] + cc * kKC);
+        for (int i = 0; i < MT; ++i) xreg[i] = load16(live ? xp[i] + c * kKC : a.x);
     };
     auto park_x = [&](int buf) {
 #pragma unroll
