@@ -188,6 +188,32 @@ def test_one_span_longer_than_64_blocks(gpu):
     check(wl, splits=2)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shapes_and_split_counts(gpu, seed):
+    """Head counts, block sizes, batch shapes (a few long, hundreds of tiny, mixed) and split-workgroup
+    counts drawn at random; sizes kept small enough for the CPU oracle."""
+    heads = [(32, 8), (16, 8), (40, 8), (8, 8), (4, 4), (12, 2), (64, 8), (16, 1), (128, 8), (32, 16)]
+    rng = np.random.default_rng(1000 + seed)
+    hq, hkv = heads[rng.integers(len(heads))]
+    bs = int(rng.choice([32, 64, 128, 256]))
+    mode = rng.integers(4)
+    if mode == 0:
+        lens = rng.integers(1, 9000, size=int(rng.integers(1, 6)))
+    elif mode == 1:
+        lens = rng.integers(1, 90, size=int(rng.integers(50, 400)))
+    elif mode == 2:
+        lens = rng.integers(1, 1500, size=int(rng.integers(8, 80)))
+    else:
+        b = int(rng.integers(2, 40))
+        lens = np.where(rng.random(b) < 0.3, rng.integers(2000, 5000, size=b), rng.integers(1, 40, size=b))
+    lens = [int(x) for x in lens]
+    while sum(lens) * hq > 2_500_000:
+        lens = lens[:-1] if len(lens) > 1 else [lens[0] // 2]
+    splits = int(rng.choice([0, 0, 1, 3, 7, 64, 200, 300, 1000]))
+    wl = workloads.make_decode_workload(f"rnd{seed}", lens, hq, hkv, bs=bs, seed=seed).to(gpu)
+    check(wl, splits=splits)
+
+
 def test_cfg2_full_size(gpu):
     wl = workloads.cfg2(device=gpu)
     err = check(wl)
