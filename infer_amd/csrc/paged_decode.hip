@@ -8,8 +8,8 @@
 //
 // Work decomposition
 //   A "step" is 32 consecutive tokens of one sequence (never straddles a cache block because
-//   block_size % 32 == 0).  All steps of all sequences are laid end to end and cut into
-//   gridDim.x equal spans; workgroup x streams span x for up to 8 KV heads, one wavefront per
+//   block_size % 32 == 0).  All steps of all sequences are laid end to end and cut into at
+//   most gridDim.x spans of equal length (to within one step); workgroup x streams span x for up to 8 KV heads, one wavefront per
 //   KV head, so a workgroup reads whole 2 KiB token rows while each wavefront runs its own
 //   private pipeline (no workgroup barrier anywhere).  A span may cover the tail of one
 //   sequence and the head of the next: each (sequence, span) piece is a "segment" and leaves a
