@@ -214,6 +214,31 @@ def test_random_shapes_and_split_counts(gpu, seed):
     check(wl, splits=splits)
 
 
+@pytest.mark.parametrize("w", [256, 100, 7])
+def test_span_count_reported_in_the_workspace_header(gpu, w):
+    """The split kernel leaves (spans used, total steps) in the first two words of the workspace.  With
+    more steps than workgroups it must use the fewest workgroups that keep the longest span at
+    ceil(total / W) steps, so no workgroup does more than the grid forces; otherwise all of them."""
+    for lens in ([4000, 77, 1300, 2048, 31, 900] * 4, [40, 33, 1], workloads.cfg2_lengths(64)):
+        wl = workloads.make_decode_workload("hdr", lens, 32, 8, seed=5).to(gpu)
+        ws = ops.decode_workspace(gpu, len(lens), 32, 8, 128)
+        prev = ops.set_split_workgroups(w)
+        try:
+            ops.paged_attn_decode_split(wl.q, wl.k_cache, wl.v_cache, wl.block_table, wl.context_lens, wl.scale, ws)
+            torch.cuda.synchronize()
+        finally:
+            ops.set_split_workgroups(prev)
+        spans, total = (int(v) for v in ws[:8].view(torch.int32)[:2].tolist())
+        assert total == sum((n + 31) // 32 for n in lens)
+        if total <= w:
+            assert spans == w
+        else:
+            longest = -(-total // w)
+            assert -(-total // spans) == longest                    # the longest span is as short as W allows
+            assert spans == w or -(-total // (spans - 1)) > longest  # and no fewer workgroups would do
+            assert spans <= w
+
+
 def test_cfg2_full_size(gpu):
     wl = workloads.cfg2(device=gpu)
     err = check(wl)
