@@ -1,6 +1,11 @@
-"""``LLMEngine`` with the interface of ``infer/engine/llm_engine.py:12-83``: ``add_request``, ``step``,
-``generate``.  A tokenizer is used when the model directory has one; without it prompts are lists of
-token ids and the outputs carry token ids only."""
+"""The request loop: ``LLMEngine.add_request`` / ``step`` / ``generate``.
+
+Interface of the reference's ``infer/engine/llm_engine.py:12-83`` (same call signatures, ``step`` returns the
+finished sequences of the step and a token count whose sign tells prefill from decode, ``generate`` returns
+one ``{"text", "token_ids"}`` record per prompt in submission order).  A tokenizer is loaded only when the
+model directory holds one: without it prompts are lists of token ids and ``text`` is ``None``.  The engine
+keeps running totals of tokens and seconds per phase in ``stats`` (the reference prints rates to a progress
+bar instead)."""
 from __future__ import annotations
 
 import os
@@ -14,23 +19,28 @@ from .scheduler import Scheduler
 from .sequence import Sequence
 
 
+def _load_tokenizer(model_dir: str):
+    if not model_dir or not os.path.exists(os.path.join(model_dir, "tokenizer.json")):
+        return None
+    from transformers import AutoTokenizer
+    return AutoTokenizer.from_pretrained(model_dir, use_fast=True)
+
+
 class LLMEngine:
 
     def __init__(self, model: str = "", **kwargs):
-        config_fields = {f.name for f in fields(Config)}
-        config = Config(model, **{k: v for k, v in kwargs.items() if k in config_fields})
-        self.config = config
-        self.model_runner = ModelRunner(config)
-        self.tokenizer = None
-        if model and os.path.exists(os.path.join(model, "tokenizer.json")):
-            from transformers import AutoTokenizer
-            self.tokenizer = AutoTokenizer.from_pretrained(model, use_fast=True)
-            config.eos = self.tokenizer.eos_token_id
-        self.scheduler = Scheduler(config)
-        self.stats = {"prefill_tokens": 0, "prefill_s": 0.0, "decode_tokens": 0, "decode_s": 0.0,
-                      "prefill_steps": 0, "decode_steps": 0}
+        known = {f.name for f in fields(Config)}
+        self.config = Config(model, **{name: value for name, value in kwargs.items() if name in known})
+        self.model_runner = ModelRunner(self.config)          # sizes the KV pool: the scheduler comes after it
+        self.tokenizer = _load_tokenizer(model)
+        if self.tokenizer is not None:
+            self.config.eos = self.tokenizer.eos_token_id
+        self.scheduler = Scheduler(self.config)
+        self.stats = dict.fromkeys(("prefill_tokens", "prefill_steps", "decode_tokens", "decode_steps"), 0)
+        self.stats.update(prefill_s=0.0, decode_s=0.0)
 
-    def add_request(self, prompt: str | list[int], sampling_params: SamplingParams):
+    # ------------------------------------------------------------------ requests
+    def add_request(self, prompt: str | list[int], sampling_params: SamplingParams) -> None:
         if isinstance(prompt, str):
             if self.tokenizer is None:
                 raise RuntimeError("a text prompt needs a tokenizer; pass token ids instead")
@@ -40,44 +50,41 @@ class LLMEngine:
     def is_finished(self) -> bool:
         return self.scheduler.is_finished()
 
+    # ------------------------------------------------------------------ one step
     def step(self):
-        seqs, is_prefill = self.scheduler.schedule()
-        token_ids = self.model_runner.run(seqs, is_prefill)
-        self.scheduler.postprocess(seqs, token_ids)
-        outputs = [(seq.seq_id, seq.completion_token_ids) for seq in seqs if seq.is_finished]
-        # a negative count marks a decode step, as in the reference
-        num_tokens = sum(len(seq) for seq in seqs) if is_prefill else -len(seqs)
-        return outputs, num_tokens
+        """Runs one scheduled step.  Returns ``(finished, count)``: ``finished`` lists ``(seq_id, completion
+        token ids)`` of the sequences that ended in this step; ``count`` is the number of prompt tokens of a
+        prefill step, or minus the number of sequences of a decode step."""
+        started = perf_counter()
+        batch, is_prefill = self.scheduler.schedule()
+        sampled = self.model_runner.run(batch, is_prefill)
+        self.scheduler.postprocess(batch, sampled)
+        count = sum(map(len, batch)) if is_prefill else -len(batch)
+        phase = "prefill" if is_prefill else "decode"
+        self.stats[phase + "_tokens"] += abs(count)
+        self.stats[phase + "_steps"] += 1
+        self.stats[phase + "_s"] += perf_counter() - started
+        finished = [(seq.seq_id, seq.completion_token_ids) for seq in batch if seq.is_finished]
+        return finished, count
 
+    # ------------------------------------------------------------------ batch interface
     def generate(self, prompts: list[str] | list[list[int]], sampling_params: SamplingParams | list[SamplingParams],
                  use_tqdm: bool = False):
-        pbar = None
+        per_prompt = sampling_params if isinstance(sampling_params, list) else [sampling_params] * len(prompts)
+        for prompt, params in zip(prompts, per_prompt):
+            self.add_request(prompt, params)
+        bar = None
         if use_tqdm:
             from tqdm.auto import tqdm
-            pbar = tqdm(total=len(prompts), desc="Generating", dynamic_ncols=True)
-        if not isinstance(sampling_params, list):
-            sampling_params = [sampling_params] * len(prompts)
-        for prompt, sp in zip(prompts, sampling_params):
-            self.add_request(prompt, sp)
-        output_dict = {}
+            bar = tqdm(total=len(prompts), desc="Generating", dynamic_ncols=True)
+        completions: dict[int, list[int]] = {}
         while not self.is_finished():
-            t = perf_counter()
-            output, num_tokens = self.step()
-            dt = perf_counter() - t
-            if num_tokens > 0:
-                self.stats["prefill_tokens"] += num_tokens
-                self.stats["prefill_s"] += dt
-                self.stats["prefill_steps"] += 1
-            else:
-                self.stats["decode_tokens"] += -num_tokens
-                self.stats["decode_s"] += dt
-                self.stats["decode_steps"] += 1
-            for seq_id, token_ids in output:
-                output_dict[seq_id] = token_ids
-                if pbar is not None:
-                    pbar.update(1)
-        if pbar is not None:
-            pbar.close()
-        outputs = [output_dict[seq_id] for seq_id in sorted(output_dict)]
-        return [{"text": self.tokenizer.decode(t) if self.tokenizer is not None else None, "token_ids": t}
-                for t in outputs]
+            finished, _ = self.step()
+            completions.update(finished)
+            if bar is not None:
+                bar.update(len(finished))
+        if bar is not None:
+            bar.close()
+        decode = self.tokenizer.decode if self.tokenizer is not None else (lambda ids: None)
+        # sequence ids grow with submission order
+        return [{"text": decode(ids), "token_ids": ids} for _, ids in sorted(completions.items())]
