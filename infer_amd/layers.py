@@ -149,9 +149,12 @@ class Sampler(nn.Module):
             # and order-preserving and argmax breaks ties by the lower index in either type, so the
             # float copy of the [batch, vocab] logits (0.4 ms per decode step at batch 128) is skipped.
             return logits.argmax(dim=-1)
-        logits = logits.to(torch.float)
-        greedy_tokens = logits.argmax(dim=-1)
-        logits.div_(temperatures.unsqueeze(dim=1))
-        probs = torch.softmax(logits, dim=-1, dtype=torch.float)
-        sample_tokens = probs.div_(torch.empty_like(probs).exponential_(1) + 1e-10).argmax(dim=-1)
-        return torch.where(temperatures == 0, greedy_tokens, sample_tokens)
+        greedy = logits.argmax(dim=-1)
+        # A draw from softmax(logits / T) as a race of exponentials: token i wins with probability p_i when
+        # the contestants are p_i / e_i with e_i ~ Exp(1).  Same arithmetic and the same consumption of the
+        # random stream as the reference (float32 throughout, 1e-10 added to the noise); rows with T = 0
+        # produce NaNs here and take the greedy token below.
+        probs = torch.softmax(logits.float() / temperatures.to(torch.float).unsqueeze(1), dim=-1)
+        noise = torch.empty_like(probs).exponential_(1.0).add_(1e-10)
+        sampled = (probs / noise).argmax(dim=-1)
+        return torch.where(temperatures == 0, greedy, sampled)
