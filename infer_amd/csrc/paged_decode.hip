@@ -75,8 +75,11 @@ __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 x) { return __builtin_bit_cast
 __device__ __forceinline__ u32x4 load16(const uint16_t* p) {
     return *reinterpret_cast<const u32x4*>(p);
 }
-// K and V rows are read once per launch: the streaming hint keeps them from displacing everything
-// else in the caches on their way through (measured on 64 sequences of 512-4096 tokens: 112.9 -> 103.4 us).
+// V rows are read once per launch, 256 contiguous bytes per token and instruction: with the streaming
+// hint the split kernel takes 103.4 instead of 112.9 us on 64 sequences of 512-4096 tokens.  K fragments
+// (64 bytes per token and instruction, each cache line touched by two instructions) gain nothing from
+// the hint, and with it the merge kernel that follows runs slower (split + merge 106.4 against 105.6 us
+// there, 175 against 170.5 us on 8 sequences of 32,768), so K is loaded plainly.
 __device__ __forceinline__ u32x4 load16_stream(const uint16_t* p) {
     return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
 }
@@ -259,7 +262,7 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) kbuf[P][t][j] = load16_stream(kb + (t * t_off + lane_off) + 32 * j);
+            for (int j = 0; j < 4; ++j) kbuf[P][t][j] = load16(kb + (t * t_off + lane_off) + 32 * j);
     };
     auto issue_v = [&]() {
         const uint16_t* vb = dummy;
