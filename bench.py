@@ -25,7 +25,7 @@ HBM_PEAK_GBS = 8000.0
 # of `python3 bench.py --counters` (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000 KiB; the factors are what
 # the same counters read for the 1 GiB plain copy run first): 631,008 KiB read + 5,057 KiB written.
 # Summary under profiles/decode_cfg2_hbm_counters.txt.  The workload is seeded, so the figure is stable.
-MEASURED_TRAFFIC_BYTES = (637348 + 4975) * 1024
+MEASURED_TRAFFIC_BYTES = (630841 + 4975) * 1024
 
 
 def gpu_time_ms(fn, iters, warmup):
