@@ -248,7 +248,7 @@ int infer_rms_norm_splitk_bf16(const float* partial, int64_t splits, int64_t spl
  * 512-thread workgroup per contiguous share) and for a copy (a grid-stride loop over `workgroups`
  * workgroups of 256 threads).  `sink4` is 4 writable bytes. */
 int infer_kv_probe_read(const void* src, size_t bytes, void* sink4, int workgroups, void* stream);
-/* the same read with the streaming (nontemporal) hint the decode kernel puts on its K and V loads */
+/* the same read with the streaming (nontemporal) hint the decode kernel puts on its V loads */
 int infer_kv_probe_read_streaming(const void* src, size_t bytes, void* sink4, int workgroups, void* stream);
 int infer_kv_probe_copy(const void* src, void* dst, size_t bytes, int workgroups, void* stream);
 /* a copy with the append kernel's launch shape: one wavefront per 4 KiB, no loop (whole 4 KiB pieces only) */

@@ -15,7 +15,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint32_t fold(u32x4 a) { return a.x ^ a.y ^ a.z ^ a.w; }
 
 // Each workgroup reads a contiguous share of the buffer exactly once.  STREAM: with the streaming
-// (nontemporal) hint the decode kernel puts on its K and V loads.
+// (nontemporal) hint the decode kernel puts on its V loads.
 template <bool STREAM>
 __device__ __forceinline__ u32x4 probe_load(const u32x4* p) { return STREAM ? __builtin_nontemporal_load(p) : *p; }
 
