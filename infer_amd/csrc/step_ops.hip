@@ -81,8 +81,9 @@ __global__ void __launch_bounds__(kNormThreads) rms_norm_kernel(NormArgs a) {
                 const float* pp = a.partial + row * a.partial_stride0 + 8 * c;
                 f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
                 for (int s = 0; s < a.splits; ++s) {
-                    lo += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(pp + s * a.split_stride));
-                    hi += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(pp + s * a.split_stride + 4));
+                    // plain loads: the two halves of a lane's 32 bytes are two instructions on the same lines
+                    lo += *reinterpret_cast<const f32x4*>(pp + s * a.split_stride);
+                    hi += *reinterpret_cast<const f32x4*>(pp + s * a.split_stride + 4);
                 }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) { v[j][e] = rb(lo[e]); v[j][4 + e] = rb(hi[e]); }
