@@ -197,8 +197,8 @@ __global__ void __launch_bounds__(256) skinny_gemm_reduce_kernel(ReduceArgs a) {
     f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
     for (int s = 0; s < a.splits; ++s) {
         const float* p = a.partial + ((int64_t)s * a.m + row) * a.n + 8 * c;
-        lo += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p));
-        hi += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p + 4));
+        lo += *reinterpret_cast<const f32x4*>(p);     // plain loads: lo and hi are two instructions on the same lines
+        hi += *reinterpret_cast<const f32x4*>(p + 4);
     }
     union { __bf16 h[8]; u32x4 u; } r;
 #pragma unroll
