@@ -8,10 +8,15 @@ uniform in [512, 4096], block tables shuffled over a pool 1.2x the need).  Input
 in HBM before the clock starts.  Successive steps walk over several independent copies of the
 cache (as successive layers of a model do) so that the 256 MB Infinity Cache cannot serve the
 reads.  Prints one JSON line.
+
+Besides the headline the line carries: the roofline of the dominant kernel, the decode op over the
+range of shapes the target names (``decode_curve``), the KV append at prefill size, the fused
+front end, the prefill attention, the CPU baselines, and the end-to-end run of the engine.
 """
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -20,12 +25,16 @@ import time
 import torch
 
 HBM_PEAK_GBS = 8000.0
+ROOT = os.path.dirname(os.path.abspath(__file__))
 
-# HBM bytes per launch of the decode split kernel on this workload, from two rocprofv3 --pmc passes
-# of `python3 bench.py --counters` (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000 KiB; the factors are what
-# the same counters read for the 1 GiB plain copy run first): 631,008 KiB read + 5,057 KiB written.
-# Summary under profiles/decode_cfg2_hbm_counters.txt.  The workload is seeded, so the figure is stable.
+# HBM bytes per launch of the decode split kernel on the headline workload.  This is a RECORDED
+# figure, not measured by this run: two `rocprofv3 --pmc` passes of `python3 bench.py --counters`
+# (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch, each scaled by what the same counter reads for the
+# 1 GiB plain copy that run launches first) gave 630,841 KiB read + 4,975 KiB written; the summary is
+# profiles/decode_cfg2_hbm_counters.txt.  The workload is seeded, so the figure only moves when the
+# kernel's access pattern does; it has to be re-recorded then.
 MEASURED_TRAFFIC_BYTES = (630841 + 4975) * 1024
+TRAFFIC_SOURCE = "recorded: profiles/decode_cfg2_hbm_counters.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)"
 
 
 def gpu_time_ms(fn, iters, warmup):
@@ -43,37 +52,104 @@ def gpu_time_ms(fn, iters, warmup):
     return start.elapsed_time(stop) / iters
 
 
-def cpu_baseline(sample_seqs=16, min_seconds=10.0):
+def load_probe_library():
+    """The measurement-only kernels (read / copy ceilings, the two halves of an append) live in a
+    library of their own, beside the product library."""
+    path = os.path.join(ROOT, "infer_amd", "libinfer_kv_probe.so")
+    if not os.path.exists(path):
+        raise ImportError(f"{path} is not built; run `make -C infer_amd/csrc`")
+    lib = ctypes.CDLL(path)
+    vp, sz, i64 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int64
+    for name, args in {
+        "infer_kv_probe_read": [vp, sz, vp, ctypes.c_int, vp],
+        "infer_kv_probe_read_streaming": [vp, sz, vp, ctypes.c_int, vp],
+        "infer_kv_probe_copy": [vp, vp, sz, ctypes.c_int, vp],
+        "infer_kv_probe_copy_rows": [vp, vp, sz, vp],
+        "infer_kv_probe_append_read_half": [vp, vp, vp, i64, i64, vp, vp],
+        "infer_kv_probe_append_write_half": [vp, vp, vp, i64, i64, vp],
+    }.items():
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = ctypes.c_int, args
+    return lib
+
+
+# ------------------------------------------------------------------------------------------ CPU legs
+def _host_threads():
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    return cores
+
+
+def _median_time(fn, min_seconds, min_runs=3, max_runs=50):
+    fn()
+    times = []
+    t_end = time.perf_counter() + min_seconds
+    while len(times) < min_runs or (time.perf_counter() < t_end and len(times) < max_runs):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    return times[len(times) // 2], len(times)
+
+
+def cpu_baseline(sample_seqs=16, min_seconds=8.0):
     """The CPU restatement of the same path (gather + SDPA, oracle/torch_path.py) on the host cores,
     over a bounded sample of the same workload: the first ``sample_seqs`` sequences of the batch."""
     from infer_amd import workloads
     from oracle import torch_path
+    cores = _host_threads()
     lengths = workloads.cfg2_lengths()[:sample_seqs]
     wl = workloads.make_decode_workload("cfg2-sample", lengths, 32, 8, seed=0, q_scale=128 ** -0.5)
-    cores = os.cpu_count() or 1
-    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
-    torch.set_num_threads(cores)
-    torch_path.paged_decode_torch(wl.q, wl.k_cache, wl.v_cache, wl.block_table, wl.context_lens, wl.scale)
-    times = []
-    t_end = time.perf_counter() + min_seconds
-    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 50):
-        t0 = time.perf_counter()
-        torch_path.paged_decode_torch(wl.q, wl.k_cache, wl.v_cache, wl.block_table, wl.context_lens, wl.scale)
-        times.append(time.perf_counter() - t0)
-    times.sort()
-    med = times[len(times) // 2]
+    med, runs = _median_time(lambda: torch_path.paged_decode_torch(wl.q, wl.k_cache, wl.v_cache, wl.block_table,
+                                                                   wl.context_lens, wl.scale), min_seconds)
     return {
         "value": round(wl.decode_bytes / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
         "sample": f"first {sample_seqs} of the 64 sequences ({sum(lengths)} tokens, "
-                  f"{wl.decode_bytes / 1e6:.1f} MB algorithmic), median of {len(times)} runs, "
+                  f"{wl.decode_bytes / 1e6:.1f} MB algorithmic), median of {runs} runs, "
                   f"torch {torch.get_num_threads()} threads",
     }
 
 
+def cpu_baselines_other(p3_cpu):
+    """The same CPU port on the other named configurations, each on a bounded sample: the whole
+    Qwen3-0.6B-shaped step (cfg1), one of the eight 32,768-token sequences of the long-context step
+    (cfg4), and the prefill-sized KV append (cfg3, ``index_copy_`` as the reference's torch path)."""
+    from infer_amd import workloads
+    from oracle import torch_path
+    cores = _host_threads()
+    out = {}
+    w1 = workloads.cfg1()
+    med, runs = _median_time(lambda: torch_path.paged_decode_torch(w1.q, w1.k_cache, w1.v_cache, w1.block_table,
+                                                                   w1.context_lens, w1.scale), 2.0)
+    out["cfg1_decode"] = {"value": round(w1.decode_bytes / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+                          "sample": f"whole step (4 sequences, {w1.decode_bytes / 1e6:.2f} MB), median of {runs} runs"}
+    w4 = workloads.make_decode_workload("cfg4-sample", [32768], 64, 8, nblk=160, seed=0)
+    med, runs = _median_time(lambda: torch_path.paged_decode_torch(w4.q, w4.k_cache, w4.v_cache, w4.block_table,
+                                                                   w4.context_lens, w4.scale), 4.0)
+    out["cfg4_decode"] = {"value": round(w4.decode_bytes / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+                          "sample": f"one of the 8 sequences of 32,768 tokens ({w4.decode_bytes / 1e6:.1f} MB), "
+                                    f"median of {runs} runs"}
+    kc, vc = p3_cpu.k_cache.clone(), p3_cpu.v_cache.clone()
+    med, runs = _median_time(lambda: torch_path.append_torch(p3_cpu.k_new, p3_cpu.v_new, kc, vc, p3_cpu.slot_mapping), 3.0)
+    out["cfg3_append"] = {"value": round(p3_cpu.append_bytes / med / 1e9, 3), "unit": "GB/s", "cores": cores,
+                          "kind": "port", "sample": f"whole step ({int(p3_cpu.slot_mapping.numel())} rows, "
+                                                    f"{p3_cpu.append_bytes / 1e6:.1f} MB), median of {runs} runs"}
+    w2 = workloads.make_decode_workload("cfg2-append", workloads.cfg2_lengths(), 32, 8, nblk=800, seed=0)
+    kc2, vc2 = w2.k_cache, w2.v_cache
+    med, runs = _median_time(lambda: torch_path.append_torch(w2.k_new, w2.v_new, kc2, vc2, w2.slot_mapping), 1.0)
+    out["cfg2_append_64_rows"] = {"value": round(med * 1e6, 2), "unit": "us", "cores": cores, "kind": "port",
+                                  "sample": f"whole step (64 rows), median of {runs} runs"}
+    return out
+
+
+# ------------------------------------------------------------------------------------------ end to end
 def run_e2e(args):
     """End-to-end decode through the engine: random-init model of a published Qwen3 shape, batch of
     random-token prompts with lengths uniform in [128, 1024], greedy decoding, KV pool filling the
-    free HBM, decode step replayed as a HIP graph.  Prints one JSON line."""
+    free HBM, decode step replayed as a HIP graph.  The first ``--e2e-check`` decode steps run twice on
+    the same state, eagerly and as the graph replay, and must sample the same tokens from finite
+    logits; at the end every cache block must be back in the pool.  Prints one JSON line."""
     import numpy as np
     from infer_amd import config as C
     from infer_amd.llm_engine import LLMEngine
@@ -88,24 +164,106 @@ def run_e2e(args):
     lengths = rng.integers(128, 1025, size=args.e2e_batch)
     prompts = [[int(t) for t in rng.integers(0, hf.vocab_size, size=int(n))] for n in lengths]
     sp = SamplingParams(temperature=0.0, max_tokens=args.e2e_new, ignore_eos=True)
+    runner = engine.model_runner
+    check = {"steps": 0, "tokens_equal": True, "logits_finite": True, "max_logit_diff": 0.0}
+    if not args.e2e_eager and args.e2e_check > 0:
+        runner.check_decode_steps = args.e2e_check      # the runner compares eager and graph on these steps
+        runner.decode_check = check
     t0 = time.perf_counter()
     outs = engine.generate(prompts, sp)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     st = engine.stats
     assert all(len(o["token_ids"]) == args.e2e_new for o in outs)
-    dec_tps = st["decode_tokens"] / st["decode_s"] if st["decode_s"] else 0.0
+    pool = engine.scheduler.block_manager
+    pool_ok = pool.num_free_blocks == engine.config.num_kvcache_blocks and len(pool.used_block_ids) == 0
+    # the checked steps stay in the count; what the check added to them (the eager run, the comparison)
+    # is taken out of the clock
+    timed_steps = st["decode_steps"]
+    timed_s = st["decode_s"] - check.get("seconds", 0.0)
+    dec_tps = st["decode_tokens"] / timed_s if timed_s else 0.0
     print(json.dumps({
         "metric": "end-to-end greedy decode throughput through the engine", "value": round(dec_tps, 1),
         "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"cfg5: random-init Qwen3-{args.e2e_model} decode, batch {args.e2e_batch}, prompts "
                                f"U[128,1024], {args.e2e_new} greedy tokens, hipGraph={not args.e2e_eager}"},
-        "decode_steps": st["decode_steps"], "decode_ms_per_step": round(1e3 * st["decode_s"] / max(st["decode_steps"], 1), 3),
+        "decode_steps": st["decode_steps"], "decode_ms_per_step": round(1e3 * timed_s / max(timed_steps, 1), 3),
+        "check_seconds_excluded": round(check.get("seconds", 0.0), 4),
         "prefill_tokens_per_s": round(st["prefill_tokens"] / st["prefill_s"], 1) if st["prefill_s"] else None,
         "prefill_steps": st["prefill_steps"], "generate_wall_s": round(wall, 2), "init_s": round(t_init, 1),
         "num_kvcache_blocks": engine.config.num_kvcache_blocks,
-        "kv_pool_GB": round(engine.model_runner.kv_cache.numel() * 2 / 1e9, 1),
-        "graphs": len(engine.model_runner.graphs)}))
+        "kv_pool_GB": round(runner.kv_cache.numel() * 2 / 1e9, 1),
+        "graphs": len(runner.graphs),
+        "checked_decode_steps": check["steps"], "tokens_equal": bool(check["tokens_equal"]) if check["steps"] else None,
+        "logits_finite": bool(check["logits_finite"]) if check["steps"] else None,
+        "max_logit_diff_eager_vs_graph": check["max_logit_diff"] if check["steps"] else None,
+        "pool_all_blocks_free_at_end": bool(pool_ok)}))
+    if check["steps"] and not (check["tokens_equal"] and check["logits_finite"]):
+        sys.exit(3)
+    if not pool_ok:
+        sys.exit(4)
+
+
+# ------------------------------------------------------------------------------------------ decode curve
+def decode_point(name, wl, copies, iters, splits=0):
+    """Decode op (split + merge) of one workload, timed as replays of a HIP graph that holds ``copies``
+    consecutive steps, each over its own copy of the caches (no host time between launches, reads
+    come from HBM)."""
+    from infer_amd import ops
+    dev = wl.q.device
+    b, hq, hkv, d = len(wl.lengths), wl.num_q_heads, wl.num_kv_heads, wl.head_dim
+    ks = [wl.k_cache] + [torch.randn_like(wl.k_cache) for _ in range(copies - 1)]
+    vs = [wl.v_cache] + [torch.randn_like(wl.v_cache) for _ in range(copies - 1)]
+    out = torch.empty((b, hq, d), dtype=torch.bfloat16, device=dev)
+    ws = ops.decode_workspace(dev, b, hq, hkv, d)
+
+    def steps():
+        for i in range(copies):
+            ops.paged_attn_decode(wl.q, ks[i], vs[i], wl.block_table, wl.context_lens, wl.scale, out, ws,
+                                  split_workgroups=splits)
+    steps()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        steps()
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            steps()
+    torch.cuda.synchronize()
+    ms = gpu_time_ms(graph.replay, iters, 2) / copies
+    nbytes = wl.decode_bytes
+    del ks, vs
+    return {"name": name, "batch": b, "Hq": hq, "tokens": sum(wl.lengths), "algorithmic_bytes": nbytes,
+            "op_us": round(ms * 1e3, 2), "GBps": round(nbytes / ms / 1e6, 1),
+            "frac_of_8TBps": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "cache_copies": copies}
+
+
+def decode_curve(dev, iters=12):
+    """The decode op over the range the target names: batch 64 at fixed context lengths 512 ... 4096
+    (Qwen3-8B heads), the long-context configuration (cfg4), and the regime the engine runs in
+    (batch 128, context lengths uniform in [128, 1280])."""
+    from infer_amd import workloads
+    points = []
+    for ctx in (512, 1024, 2048, 4096):
+        wl = workloads.make_decode_workload(f"b64-ctx{ctx}", [ctx] * 64, 32, 8, seed=ctx, q_scale=128 ** -0.5,
+                                            device=dev, device_fill=True)
+        pool_mb = 2 * wl.k_cache.numel() * 2 / 1e6
+        points.append(decode_point(f"batch 64 x ctx {ctx}", wl, max(2, min(8, int(1100 / pool_mb) + 1)), iters))
+        del wl
+        torch.cuda.empty_cache()
+    gen = torch.Generator().manual_seed(5)
+    lens = torch.randint(128, 1281, (128,), generator=gen).tolist()
+    wl = workloads.make_decode_workload("b128-engine", lens, 32, 8, seed=5, q_scale=128 ** -0.5, device=dev,
+                                        device_fill=True)
+    points.append(decode_point("batch 128 x ctx U[128,1280] (engine regime)", wl, 4, iters))
+    del wl
+    torch.cuda.empty_cache()
+    wl = workloads.cfg4(device=dev, device_fill=True)
+    points.append(decode_point("cfg4: batch 8 x ctx 32768, Hq=64", wl, 2, iters))
+    del wl
+    torch.cuda.empty_cache()
+    return points
 
 
 def main():
@@ -114,22 +272,26 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--copies", type=int, default=4, help="independent cache copies walked round-robin")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--splits", type=int, default=0, help="KV-split workgroups (0 = library default)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--no-curve", action="store_true", help="skip the decode curve of the default run")
+    ap.add_argument("--splits", type=int, default=0, help="KV-split workgroups per decode call (0 = library default)")
     ap.add_argument("--ceiling", action="store_true",
                     help="measure what this GPU sustains for a read-only stream and a copy (plain kernels of the "
-                         "library, same timing method) and print it as JSON; no KV-cache kernel runs")
+                         "probe library, same timing method) and print it as JSON; no KV-cache kernel runs")
     ap.add_argument("--counters", action="store_true",
                     help="short untimed run for `rocprofv3 --pmc`: a 1 GiB plain copy (x3), the decode op (x5), "
-                         "a prefill-sized append (x3)")
+                         "a prefill-sized append (x3), its read half and its write half (x3 each)")
     ap.add_argument("--append-sweep", action="store_true",
                     help="KV append rate against the number of rows (64 ... 65,536), printed as JSON")
+    ap.add_argument("--decode-curve", action="store_true", help="only the decode curve, printed as JSON")
     ap.add_argument("--e2e", action="store_true",
                     help="end-to-end decode through the engine (random-init Qwen3, HIP-graph decode) instead "
                          "of the kernel benchmark")
     ap.add_argument("--e2e-model", default="8b", choices=["0.6b", "8b", "32b"])
     ap.add_argument("--e2e-batch", type=int, default=128)
     ap.add_argument("--e2e-new", type=int, default=256)
+    ap.add_argument("--e2e-check", type=int, default=8,
+                    help="decode steps at the start that run both eagerly and as graph replays and are compared")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end leg of the default run")
     ap.add_argument("--e2e-eager", action="store_true", help="run the decode steps eagerly (no HIP graph)")
     args = ap.parse_args()
@@ -144,11 +306,10 @@ def main():
     if args.e2e:
         run_e2e(args)
         return
-    from infer_amd import ops, workloads
+    from infer_amd import _lib, ops, workloads
     dev = torch.device("cuda:0")
     if args.ceiling:
-        from infer_amd import _lib
-        lib = _lib.load()
+        lib = load_probe_library()
         stream = torch.cuda.current_stream().cuda_stream
         sink = torch.zeros(4, dtype=torch.uint8, device=dev)
         res = {"ceiling_run": True, "method": "HIP events, 30 launches after 3 warm-ups, buffers rotated (4 x size)"}
@@ -170,12 +331,14 @@ def main():
                     it[0] += 1
                     _lib.check(lib.infer_kv_probe_copy(bufs[i].data_ptr(), dst.data_ptr(), nbytes, wg, stream), "probe")
                 return f
+
             def rds(wg):
                 def f():
                     i = it[0] % 4
                     it[0] += 1
                     _lib.check(lib.infer_kv_probe_read_streaming(bufs[i].data_ptr(), nbytes, sink.data_ptr(), wg, stream), "probe")
                 return f
+
             def cprows():
                 i = it[0] % 4
                 it[0] += 1
@@ -204,7 +367,7 @@ def main():
         pool_rows = 1 << 18
         caches = [(torch.empty((pool_rows // 256, 256, 8, 128), dtype=torch.bfloat16, device=dev),
                    torch.empty((pool_rows // 256, 256, 8, 128), dtype=torch.bfloat16, device=dev)) for _ in range(2)]
-        for n in (64, 256, 1024, 4096, 16384, 65536):
+        for n in (64, 256, 1024, 2048, 3072, 4096, 8192, 16384, 32768, 65536):
             reps = max(2, min(16, (600 << 20) // (n * 4 * dkv)))
             srcs = [(torch.randn((n, 8, 128), dtype=torch.bfloat16, device=dev),
                      torch.randn((n, 8, 128), dtype=torch.bfloat16, device=dev)) for _ in range(reps)]
@@ -247,16 +410,23 @@ def main():
             del srcs, layouts
         print(json.dumps(res))
         return
-    if args.splits:
-        ops.set_split_workgroups(args.splits)
-    wl = workloads.cfg2(device=dev)
-    b, hq, hkv, d = len(wl.lengths), wl.num_q_heads, wl.num_kv_heads, wl.head_dim
+    if args.decode_curve:
+        print(json.dumps({"decode_curve": decode_curve(dev)}))
+        return
+
+    p3_cpu = workloads.cfg3()                       # drawn on the CPU from the seed; also the CPU append baseline
     if args.counters:
+        wl = workloads.cfg2(device=dev, device_fill=True)
+        b, hq, hkv, d = len(wl.lengths), wl.num_q_heads, wl.num_kv_heads, wl.head_dim
+        probe = load_probe_library()
+        stream = torch.cuda.current_stream().cuda_stream
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
         dst = torch.empty_like(src)
         out = torch.empty((b, hq, d), dtype=torch.bfloat16, device=dev)
         ws = ops.decode_workspace(dev, b, hq, hkv, d)
-        p3 = workloads.cfg3(device=dev)
+        p3 = p3_cpu.to(dev)
+        sink = torch.zeros(4, dtype=torch.uint8, device=dev)
+        n3, slots3 = int(p3.slot_mapping.numel()), p3.k_cache.shape[0] * 256
         torch.cuda.synchronize()
         for _ in range(3):
             dst.copy_(src)      # plain copy of known size: 1 GiB read, 1 GiB written
@@ -264,10 +434,20 @@ def main():
             ops.paged_attn_decode(wl.q, wl.k_cache, wl.v_cache, wl.block_table, wl.context_lens, wl.scale, out, ws)
         for _ in range(3):
             ops.store_kvcache(p3.k_new, p3.v_new, p3.k_cache, p3.v_cache, p3.slot_mapping)
+        for _ in range(3):
+            _lib.check(probe.infer_kv_probe_append_read_half(p3.k_new.data_ptr(), p3.v_new.data_ptr(),
+                                                             p3.slot_mapping.data_ptr(), n3, slots3, sink.data_ptr(),
+                                                             stream), "probe")
+        for _ in range(3):
+            _lib.check(probe.infer_kv_probe_append_write_half(p3.k_cache.data_ptr(), p3.v_cache.data_ptr(),
+                                                              p3.slot_mapping.data_ptr(), n3, slots3, stream), "probe")
         torch.cuda.synchronize()
         print(json.dumps({"counters_run": True, "copy_bytes": 1 << 30, "decode_algorithmic_bytes": wl.decode_bytes,
                           "append_algorithmic_bytes": p3.append_bytes}))
         return
+
+    wl = workloads.cfg2().to(dev)                   # the headline workload: seeded on the CPU, then moved
+    b, hq, hkv, d = len(wl.lengths), wl.num_q_heads, wl.num_kv_heads, wl.head_dim
     k_copies = [wl.k_cache] + [torch.randn_like(wl.k_cache) for _ in range(args.copies - 1)]
     v_copies = [wl.v_cache] + [torch.randn_like(wl.v_cache) for _ in range(args.copies - 1)]
     out = torch.empty((b, hq, d), dtype=torch.bfloat16, device=dev)
@@ -277,12 +457,14 @@ def main():
     def step():
         i = it[0] % args.copies
         it[0] += 1
-        ops.paged_attn_decode(wl.q, k_copies[i], v_copies[i], wl.block_table, wl.context_lens, wl.scale, out, ws)
+        ops.paged_attn_decode(wl.q, k_copies[i], v_copies[i], wl.block_table, wl.context_lens, wl.scale, out, ws,
+                              split_workgroups=args.splits)
 
     def split_only():
         i = it[0] % args.copies
         it[0] += 1
-        ops.paged_attn_decode_split(wl.q, k_copies[i], v_copies[i], wl.block_table, wl.context_lens, wl.scale, ws)
+        ops.paged_attn_decode_split(wl.q, k_copies[i], v_copies[i], wl.block_table, wl.context_lens, wl.scale, ws,
+                                    split_workgroups=args.splits)
 
     # whole op, exactly K steps
     for _ in range(args.warmup):
@@ -305,7 +487,7 @@ def main():
     # KV append: decode-sized (64 rows, latency bound) and prefill-sized (cfg3)
     ap_small_ms = gpu_time_ms(lambda: ops.store_kvcache(wl.k_new, wl.v_new, wl.k_cache, wl.v_cache, wl.slot_mapping),
                               args.steps, 5)
-    p3 = workloads.cfg3(device=dev)
+    p3 = p3_cpu.to(dev)
     reps = 24   # distinct source/destination buffers walked round-robin (24 x ~100 MB > Infinity Cache)
     srcs = [(torch.randn_like(p3.k_new), torch.randn_like(p3.v_new)) for _ in range(reps)]
     dsts = [(torch.empty_like(p3.k_cache), torch.empty_like(p3.v_cache)) for _ in range(reps)]
@@ -318,20 +500,48 @@ def main():
 
     ap_ms = gpu_time_ms(append_step, max(args.steps, 48), reps)
     append_gbs = p3.append_bytes / (ap_ms * 1e-3) / 1e9
+    # the two halves of that append on their own (probe library): what its reads and its writes cost alone
+    probe = load_probe_library()
+    stream = torch.cuda.current_stream().cuda_stream
+    sink = torch.zeros(4, dtype=torch.uint8, device=dev)
+    n3, slots3 = int(p3.slot_mapping.numel()), p3.k_cache.shape[0] * 256
 
-    # fused QK-norm + RoPE + append (one launch for the four steps in front of attention)
+    def read_half():
+        j = jt[0] % reps
+        jt[0] += 1
+        probe.infer_kv_probe_append_read_half(srcs[j][0].data_ptr(), srcs[j][1].data_ptr(), p3.slot_mapping.data_ptr(),
+                                              n3, slots3, sink.data_ptr(), stream)
+
+    def write_half():
+        j = jt[0] % reps
+        jt[0] += 1
+        probe.infer_kv_probe_append_write_half(dsts[j][0].data_ptr(), dsts[j][1].data_ptr(), p3.slot_mapping.data_ptr(),
+                                               n3, slots3, stream)
+    rd_ms = gpu_time_ms(read_half, 48, reps)
+    wr_ms = gpu_time_ms(write_half, 48, reps)
+
+    # fused QK-norm + RoPE + append (one launch for the four steps in front of attention), over rotated
+    # qkv buffers and cache pairs (> 512 MB in total) so that every launch reads and writes HBM
     def fused_case(n_rows):
         d_ = 128
-        qkv = torch.randn((n_rows, (hq + 2 * hkv) * d_), dtype=torch.bfloat16, device=dev)
-        q_, k_, v_ = (t.view(n_rows, -1, d_) for t in qkv.split([hq * d_, hkv * d_, hkv * d_], dim=-1))
+        row = (hq + 2 * hkv) * d_
+        nbuf = max(2, min(reps, (700 << 20) // (n_rows * row * 2) + 1))
+        qkvs = [torch.randn((n_rows, row), dtype=torch.bfloat16, device=dev) for _ in range(nbuf)]
         w_ = torch.ones(d_, dtype=torch.bfloat16, device=dev)
         cs_ = torch.randn((4096, d_), dtype=torch.bfloat16, device=dev)
         pos_ = torch.randint(0, 4096, (n_rows,), device=dev)
         sl_ = torch.randperm(p3.k_cache.shape[0] * 256, device=dev)[:n_rows].to(torch.int32)
-        ms_ = gpu_time_ms(lambda: ops.qk_norm_rope_store_kvcache(q_, k_, v_, pos_, w_, w_, 1e-6, cs_, dsts[0][0],
-                                                                 dsts[0][1], sl_), 50, 5)
-        nbytes_ = n_rows * (2 * hq * d_ * 2 + 5 * hkv * d_ * 2)   # q r+w, k r+w+cache, v r+cache
-        return round(ms_ * 1e3, 2), round(nbytes_ / ms_ / 1e6, 1)
+        ft = [0]
+
+        def fused_step():
+            j = ft[0]
+            ft[0] += 1
+            q_, k_, v_ = (t.view(n_rows, -1, d_) for t in qkvs[j % nbuf].split([hq * d_, hkv * d_, hkv * d_], dim=-1))
+            kc_, vc_ = dsts[j % reps]
+            ops.qk_norm_rope_store_kvcache(q_, k_, v_, pos_, w_, w_, 1e-6, cs_, kc_, vc_, sl_, write_key=False)
+        ms_ = gpu_time_ms(fused_step, 48, 6)
+        nbytes_ = n_rows * (2 * hq * d_ * 2 + 4 * hkv * d_ * 2)   # q read + written in place, k and v read, both stored
+        return round(ms_ * 1e3, 2), round(nbytes_ / ms_ / 1e6, 1), nbuf
     fused_small = fused_case(b)
     fused_big = fused_case(int(p3.q.shape[0]))
 
@@ -357,11 +567,13 @@ def main():
         "wall_ms_per_step": round(wall_ms, 5),
         "roofline": {"bound": "hbm", "kernel": "paged_decode_split_kernel", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES, "avg_kernel_ms": round(split_ms, 5)},
+                     "traffic": MEASURED_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE,
+                     "avg_kernel_ms": round(split_ms, 5)},
         "append": {"decode_rows": b, "decode_us": round(ap_small_ms * 1e3, 2),
                    "prefill_rows": int(p3.slot_mapping.numel()), "prefill_bytes": p3.append_bytes,
                    "prefill_us": round(ap_ms * 1e3, 2), "prefill_GBps": round(append_gbs, 1),
-                   "prefill_frac_of_peak": round(append_gbs / HBM_PEAK_GBS, 4)},
+                   "prefill_frac_of_peak": round(append_gbs / HBM_PEAK_GBS, 4),
+                   "read_half_alone_us": round(rd_ms * 1e3, 2), "write_half_alone_us": round(wr_ms * 1e3, 2)},
     }
     line["prefill_attention"] = {"workload": "cfg3: 16 prompts U[64,2048], 0-50 % cached, causal over the paged cache",
                                  "query_tokens": int(p3.q.shape[0]), "ms": round(pf_ms, 4),
@@ -369,14 +581,21 @@ def main():
     line["fused_qk_norm_rope_append"] = {"decode_rows": b, "decode_us": fused_small[0],
                                          "prefill_rows": int(p3.q.shape[0]), "prefill_us": fused_big[0],
                                          "prefill_GBps": fused_big[1],
-                                         "note": "same 161 MB qkv buffer every launch: partly served by the "
-                                                 "256 MB Infinity Cache, not an HBM figure"}
+                                         "prefill_frac_of_peak": round(fused_big[1] / HBM_PEAK_GBS, 4),
+                                         "note": f"{fused_big[2]} qkv buffers and {reps} cache pairs walked round-robin "
+                                                 "(> 512 MB): an HBM figure; bytes = q in + q out + k in + v in + "
+                                                 "k and v stored"}
+    del k_copies, v_copies, srcs, dsts, kc3, vc3
+    torch.cuda.empty_cache()
+    if not args.no_curve:
+        line["decode_curve"] = decode_curve(dev)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline()
+        line["cpu_baselines_other_configs"] = cpu_baselines_other(p3_cpu)
     if not args.no_e2e:
         # the end-to-end configuration runs in a child process of its own (it sizes its KV pool from the
         # free HBM); its JSON line is attached as a secondary figure and never affects `value`
-        del k_copies, v_copies, srcs, dsts, kc3, vc3
+        del wl, p3, out, ws
         torch.cuda.empty_cache()
         import subprocess
         try:

@@ -100,17 +100,25 @@ int infer_kv_qk_norm_rope_append_bf16(void* q, int64_t q_stride0, void* k, int64
  *
  * Rows with context_lens[b] <= 0 (graph padding) write zeros.  Table entries past
  * ceil(len / block_size) are never read; entries that are read are clamped into
- * [0, num_blocks) so a corrupt table cannot fault the GPU.
+ * [0, num_blocks) so a corrupt table cannot fault the GPU, and a length beyond what a table row can
+ * address (table_cols * block_size) is cut to that, so a corrupt length cannot make the gather run
+ * past its row.
  *
  * Layouts (strides in elements): q [B, Hq, D] with row stride q_stride0, heads contiguous;
  * out likewise with out_stride0; caches [num_blocks, block_size, Hkv, D] with block stride
  * cache_block_stride and token stride cache_token_stride (heads contiguous, D innermost);
- * block_table [B, *] with row stride bt_stride0; context_lens [B].
+ * block_table [B, table_cols] with row stride bt_stride0 >= table_cols; context_lens [B].
  *
  * The work is split across workgroups in equal shares of KV tokens regardless of sequence
  * boundaries; partial (max, sum, accumulator) results go to `workspace` and are merged by a
  * second small kernel.  Size the workspace with infer_paged_decode_workspace_bytes() for the
- * largest batch that will be passed; its contents need no initialisation.
+ * largest batch that will be passed; its contents need no initialisation.  Calls that share a
+ * workspace must be ordered on one stream (the records of one call are live until its merge kernel
+ * has run); calls on different streams need a workspace each.
+ *
+ * split_workgroups: workgroups along the KV-split axis of this call, 0 = choose from the device's
+ * compute-unit count (the tuned default), at most 1024.  The library keeps no state between calls:
+ * two calls may use different counts, also concurrently.
  *
  * Built for head_dim == 128, 1 <= G <= 16, block_size % 32 == 0 (the reference requires a
  * multiple of 256: infer/config.py:21), num_kv_heads <= 8 or a multiple of 8.
@@ -122,26 +130,27 @@ int infer_paged_decode_bf16(const void* q, int64_t q_stride0,
                             const void* k_cache, const void* v_cache,
                             int64_t cache_block_stride, int64_t cache_token_stride,
                             void* out, int64_t out_stride0,
-                            const int32_t* block_table, int64_t bt_stride0,
+                            const int32_t* block_table, int64_t bt_stride0, int64_t table_cols,
                             const int32_t* context_lens,
                             int64_t batch, int64_t num_q_heads, int64_t num_kv_heads,
                             int64_t head_dim, int64_t block_size, int64_t num_blocks,
-                            float scale,
+                            float scale, int64_t split_workgroups,
                             void* workspace, size_t workspace_bytes,
                             void* stream);
 
-/* The two phases of infer_paged_decode_bf16 on their own (same arguments): `split` streams the
- * KV cache and leaves partial results in the workspace, `merge` combines them into `out`.
- * Calling split then merge on one stream is exactly infer_paged_decode_bf16.  They exist so a
- * profiler or a benchmark can time the bandwidth-bound phase alone. */
+/* The two phases of infer_paged_decode_bf16 on their own: `split` streams the KV cache and leaves
+ * partial results in the workspace, `merge` combines them into `out`.  Calling split then merge
+ * on one stream is exactly infer_paged_decode_bf16.  They exist so a profiler or a benchmark can
+ * time the bandwidth-bound phase alone.  The merge finds the records from the workspace alone, so
+ * it does not need to know the split count. */
 int infer_paged_decode_split_bf16(const void* q, int64_t q_stride0,
                                   const void* k_cache, const void* v_cache,
                                   int64_t cache_block_stride, int64_t cache_token_stride,
-                                  const int32_t* block_table, int64_t bt_stride0,
+                                  const int32_t* block_table, int64_t bt_stride0, int64_t table_cols,
                                   const int32_t* context_lens,
                                   int64_t batch, int64_t num_q_heads, int64_t num_kv_heads,
                                   int64_t head_dim, int64_t block_size, int64_t num_blocks,
-                                  float scale,
+                                  float scale, int64_t split_workgroups,
                                   void* workspace, size_t workspace_bytes,
                                   void* stream);
 
@@ -166,22 +175,21 @@ int infer_paged_decode_merge_bf16(void* out, int64_t out_stride0,
  * kv_rows = number of token rows addressable through k/v (packed: rows of the tensor; paged:
  * num_blocks * block_size); it only bounds reads.  causal != 0 applies the bottom-right aligned
  * mask (key j visible to query i of the sequence iff j <= i + (sk - sq)).  Queries of a sequence
- * with sk == 0 produce zeros.  Same shape limits as the decode entry points.  No workspace.
+ * with sk == 0 produce zeros.  With a block table, table_cols is the number of entries per row
+ * (bt_stride0 >= table_cols) and a key length beyond table_cols * block_size is cut to that.  scale
+ * must be positive (INFER_KV_EINVAL otherwise).  Same shape limits as the decode entry points.  No
+ * workspace.
  */
 int infer_paged_prefill_bf16(const void* q, int64_t q_stride0,
                              const void* k, const void* v,
                              int64_t kv_block_stride, int64_t kv_token_stride, int64_t kv_rows,
                              void* out, int64_t out_stride0,
                              const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
-                             const int32_t* block_table, int64_t bt_stride0,
+                             const int32_t* block_table, int64_t bt_stride0, int64_t table_cols,
                              int64_t num_seqs, int64_t max_seqlen_q,
                              int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
                              int64_t block_size, int64_t num_blocks,
                              float scale, int causal, void* stream);
-
-/* Tuning knob: number of workgroups along the KV-split axis used by the decode kernels
- * (0 = choose from the device's CU count).  Process-wide; returns the previous value. */
-int infer_paged_decode_set_split_workgroups(int workgroups);
 
 /* ------------------------------------------------------------------ 2c. the operators of a decode step around the path
  * What the engine runs between two attention calls of a captured decode step, so that the step is
@@ -241,18 +249,6 @@ int infer_rms_norm_splitk_bf16(const float* partial, int64_t splits, int64_t spl
                                int64_t partial_stride0, void* residual, int64_t residual_stride0,
                                const void* weight, void* out, int64_t out_stride0,
                                int64_t n_rows, int64_t hidden, float eps, void* stream);
-
-/* ------------------------------------------------------------------ measurement helpers
- * No counterpart in the reference.  Plain streaming kernels used by bench.py --ceiling to measure
- * what the part sustains for a read-only stream (same launch shape as the decode kernel: one
- * 512-thread workgroup per contiguous share) and for a copy (a grid-stride loop over `workgroups`
- * workgroups of 256 threads).  `sink4` is 4 writable bytes. */
-int infer_kv_probe_read(const void* src, size_t bytes, void* sink4, int workgroups, void* stream);
-/* the same read with the streaming (nontemporal) hint the decode kernel puts on its V loads */
-int infer_kv_probe_read_streaming(const void* src, size_t bytes, void* sink4, int workgroups, void* stream);
-int infer_kv_probe_copy(const void* src, void* dst, size_t bytes, int workgroups, void* stream);
-/* a copy with the append kernel's launch shape: one wavefront per 4 KiB, no loop (whole 4 KiB pieces only) */
-int infer_kv_probe_copy_rows(const void* src, void* dst, size_t bytes, void* stream);
 
 /* ------------------------------------------------------------------ 3. block pool (host only)
  * C view of infer::BlockPool (include/infer_kv/block_pool.hpp), the native counterpart of the

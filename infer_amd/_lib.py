@@ -27,14 +27,13 @@ SIGNATURES = {
     "infer_kv_qk_norm_rope_append_bf16": (_c.c_int, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _f32, _vp, _i64,
                                                      _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _c.c_int, _vp]),
     "infer_paged_decode_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64]),
-    "infer_paged_decode_bf16": (_c.c_int, [_vp, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _i64, _vp,
-                                           _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp, _sz, _vp]),
-    "infer_paged_decode_split_bf16": (_c.c_int, [_vp, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _vp,
-                                                 _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp, _sz, _vp]),
+    "infer_paged_decode_bf16": (_c.c_int, [_vp, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _vp,
+                                           _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _vp, _sz, _vp]),
+    "infer_paged_decode_split_bf16": (_c.c_int, [_vp, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _vp,
+                                                 _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _vp, _sz, _vp]),
     "infer_paged_decode_merge_bf16": (_c.c_int, [_vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _sz, _vp]),
-    "infer_paged_decode_set_split_workgroups": (_c.c_int, [_c.c_int]),
     "infer_paged_prefill_bf16": (_c.c_int, [_vp, _i64, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _i64,
-                                            _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _c.c_int, _vp]),
+                                            _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _c.c_int, _vp]),
     "infer_rms_norm_bf16": (_c.c_int, [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _f32, _vp]),
     "infer_silu_and_mul_bf16": (_c.c_int, [_vp, _i64, _vp, _i64, _i64, _i64, _vp]),
     "infer_decode_metadata": (_c.c_int, [_vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
@@ -43,10 +42,6 @@ SIGNATURES = {
     "infer_skinny_gemm_partial_bf16": (_c.c_int, [_vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _sz, _vp, _vp]),
     "infer_rms_norm_splitk_bf16": (_c.c_int, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _f32,
                                               _vp]),
-    "infer_kv_probe_read": (_c.c_int, [_vp, _sz, _vp, _c.c_int, _vp]),
-    "infer_kv_probe_read_streaming": (_c.c_int, [_vp, _sz, _vp, _c.c_int, _vp]),
-    "infer_kv_probe_copy": (_c.c_int, [_vp, _vp, _sz, _c.c_int, _vp]),
-    "infer_kv_probe_copy_rows": (_c.c_int, [_vp, _vp, _sz, _vp]),
     "infer_pool_create": (_vp, [_i32, _i32]),
     "infer_pool_destroy": (None, [_vp]),
     "infer_pool_last_error": (_c.c_char_p, []),

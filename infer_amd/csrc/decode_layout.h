@@ -5,8 +5,9 @@
 
 #include "../../include/infer_kv.h"
 
-// Upper bound on the number of KV-split workgroups; the workspace is always laid out for it, so
-// its offsets do not depend on the tuning knob.
+// Upper bound on the number of KV-split workgroups.  A caller-provided workspace is always laid out
+// for it, so its offsets depend on nothing but the shape: the split and the merge launch agree on
+// where every record lives whatever split count a call asks for.
 #define INFER_KV_MAX_SPLIT_WG 1024
 
 struct DecodeWorkspace {
@@ -15,6 +16,7 @@ struct DecodeWorkspace {
     size_t seg_last_off;    // int32[batch]: last one
     size_t rec_off;         // [slots] records of rec_stride bytes, one per (segment, KV head)
     size_t rec_stride;      // bytes per record, a multiple of 16
+    int64_t slots_per_head; // records per KV head: split_cap + batch
     size_t total_bytes;
 };
 
@@ -27,12 +29,16 @@ static inline size_t align_up_256(size_t x) { return (x + 255) & ~(size_t)255; }
 // padded to a multiple of 16 bytes.
 static inline size_t decode_record_bytes(int64_t group) { return ((size_t)group * 520 + 15) & ~(size_t)15; }
 
-// slots = num_kv_heads * (INFER_KV_MAX_SPLIT_WG + batch): segment (workgroup w, sequence b) of KV
-// head h uses slot h * (W + batch) + w + b, which is unique because consecutive segments along
-// the flattened token axis advance w or b (or both) by one.
-static inline DecodeWorkspace decode_workspace_layout(int64_t batch, int64_t group, int64_t num_kv_heads) {
+// slots = num_kv_heads * (split_cap + batch): segment (workgroup w < split_cap, sequence b) of KV
+// head h uses slot h * (split_cap + batch) + w + b, which is unique because consecutive segments
+// along the flattened token axis advance w or b (or both) by one.  split_cap is
+// INFER_KV_MAX_SPLIT_WG for a caller-provided workspace; the entry point that brings its own
+// fixed-size scratch lays it out for the split count it launches.
+static inline DecodeWorkspace decode_workspace_layout(int64_t batch, int64_t group, int64_t num_kv_heads,
+                                                      int64_t split_cap = INFER_KV_MAX_SPLIT_WG) {
     DecodeWorkspace ws;
-    const size_t slots = (size_t)num_kv_heads * (size_t)(INFER_KV_MAX_SPLIT_WG + batch);
+    ws.slots_per_head = split_cap + batch;
+    const size_t slots = (size_t)num_kv_heads * (size_t)ws.slots_per_head;
     size_t off = 0;
     ws.header_off = off;      off = align_up_256(off + 64 * sizeof(int32_t));
     ws.seg_first_off = off;   off = align_up_256(off + (size_t)batch * sizeof(int32_t));

@@ -56,6 +56,7 @@ struct DecodeArgs {
     const int32_t* bt;
     int64_t bt_stride0;
     const int32_t* ctx;
+    int max_ctx;        // lengths are clamped to what the block table can address (table_cols * block_size)
     int batch;
     int group;          // query heads per KV head
     int num_kv_heads;
@@ -67,7 +68,7 @@ struct DecodeArgs {
     int32_t* seg_last;
     unsigned char* rec; // [slots] partial-result records (layout: decode_record_bytes)
     int rec_stride;
-    int slots_per_head; // gridDim.x + batch
+    int slots_per_head; // records per KV head in the workspace (layout constant, >= gridDim.x + batch)
 };
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 x) { return __builtin_bit_cast(bf16x8, x); }
@@ -85,6 +86,13 @@ __device__ __forceinline__ u32x4 load16_stream(const uint16_t* p) {
 }
 
 __device__ __forceinline__ int steps_of(int len) { return len > 0 ? (len + kStep - 1) / kStep : 0; }
+
+// Context length of sequence i as the kernels use it: a length the block table row cannot address is
+// cut to the row's capacity, so a corrupt length cannot make the table gather run past the row.
+__device__ __forceinline__ int ctx_len(const int32_t* ctx, int max_ctx, int i) {
+    const int len = ctx[i];
+    return len < max_ctx ? len : max_ctx;
+}
 
 // Inclusive prefix sum over the 64 lanes on the vector pipe (data-parallel primitives): shifts by 1,
 // 2, 4 and 8 inside each row of 16 lanes, then the last lane of row 0 (2) is added to row 1 (3) and the
@@ -441,11 +449,11 @@ __global__ void __launch_bounds__(512) paged_decode_split_kernel(DecodeArgs a) {
     const int steps_per_blk = a.block_size / kStep;
 
     // total number of steps (the first 64 lengths stay in registers for the second pass)
-    const int len0 = lane < a.batch ? a.ctx[lane] : 0;
+    const int len0 = lane < a.batch ? ctx_len(a.ctx, a.max_ctx, lane) : 0;
     int total = wave_sum(steps_of(len0));
     for (int c = 64; c < a.batch; c += 64) {
         const int i = c + lane;
-        total += wave_sum(i < a.batch ? steps_of(a.ctx[i]) : 0);
+        total += wave_sum(i < a.batch ? steps_of(ctx_len(a.ctx, a.max_ctx, i)) : 0);
     }
     total = __builtin_amdgcn_readfirstlane(total);   // wave-uniform: keep the plan in scalar registers
 
@@ -478,7 +486,7 @@ __global__ void __launch_bounds__(512) paged_decode_split_kernel(DecodeArgs a) {
     int running = 0;
     for (int c = 0; c < a.batch; c += 64) {
         const int i = c + lane;
-        const int len = c == 0 ? len0 : (i < a.batch ? a.ctx[i] : 0);
+        const int len = c == 0 ? len0 : (i < a.batch ? ctx_len(a.ctx, a.max_ctx, i) : 0);
         const int cnt = steps_of(len);
         const int incl = wave_inclusive_scan(cnt, lane);
         const int start = running + incl - cnt;
@@ -532,7 +540,7 @@ struct MergeArgs {
     int64_t out_stride0;
     const int32_t* ctx;
     int group;
-    int split_workgroups;   // gridDim.x of the split launch that filled the workspace
+    int slots_per_head;     // records per KV head in the workspace, as in the split launch
     const int32_t* seg_first;
     const int32_t* seg_last;
     const unsigned char* rec;
@@ -557,7 +565,7 @@ __global__ void __launch_bounds__(256) paged_decode_merge_kernel(MergeArgs a) {
         return;
     }
     const int w0 = a.seg_first[b], w1 = a.seg_last[b];
-    const int64_t slot0 = (int64_t)h * (a.split_workgroups + a.batch) + b;
+    const int64_t slot0 = (int64_t)h * a.slots_per_head + b;
     float m = -INFINITY, den = 0.f;
     f32x4 num = {0.f, 0.f, 0.f, 0.f};
     for (int wb = w0 + j; wb <= w1; wb += 32) {
@@ -606,8 +614,6 @@ __global__ void __launch_bounds__(256) paged_decode_merge_kernel(MergeArgs a) {
     }
 }
 
-int g_split_workgroups = 0;
-
 constexpr int kMaxDevices = 64;
 
 int current_device() {
@@ -631,34 +637,133 @@ int device_cu_count() {
 struct Launch {
     int waves;      // wavefronts (KV heads) per workgroup
     int grid_y;
-    int W;
+    int W;          // workgroups along the KV-split axis
 };
 
-int plan_launch(int64_t hkv, Launch* out) {
-    if (hkv <= 0) return INFER_KV_EINVAL;
+// split_workgroups: 0 = two wavefronts per SIMD over the whole chip, else the caller's count.
+int plan_launch(int64_t hkv, int64_t split_workgroups, Launch* out) {
+    if (hkv <= 0 || split_workgroups < 0) return INFER_KV_EINVAL;
     int waves;
     if (hkv <= 8) waves = (int)hkv;
     else if (hkv % 8 == 0) waves = 8;
     else return INFER_KV_EUNSUPPORTED;
-    int W = g_split_workgroups;
-    if (W <= 0) {
-        W = device_cu_count() * 8 / (int)hkv;   // two wavefronts per SIMD over the whole chip
+    int64_t W = split_workgroups;
+    if (W == 0) {
+        W = device_cu_count() * 8 / hkv;
         if (W < 1) W = 1;
     }
     if (W > INFER_KV_MAX_SPLIT_WG) W = INFER_KV_MAX_SPLIT_WG;
     out->waves = waves;
     out->grid_y = (int)(hkv / waves);
-    out->W = W;
+    out->W = (int)W;
     return INFER_KV_OK;
 }
 
-int check_shape(int64_t batch, int64_t hq, int64_t hkv, int64_t d, int64_t bs, int64_t nblk) {
-    if (batch <= 0 || hq <= 0 || hkv <= 0 || nblk <= 0 || bs <= 0) return INFER_KV_EINVAL;
+int check_shape(int64_t batch, int64_t hq, int64_t hkv, int64_t d, int64_t bs, int64_t nblk, int64_t table_cols) {
+    if (batch <= 0 || hq <= 0 || hkv <= 0 || nblk <= 0 || bs <= 0 || table_cols <= 0) return INFER_KV_EINVAL;
     if (batch > (1 << 20)) return INFER_KV_EINVAL;
     if (d != kD) return INFER_KV_EUNSUPPORTED;
     if (hq % hkv != 0 || hq / hkv > 16) return INFER_KV_EUNSUPPORTED;
     if (bs % kStep != 0) return INFER_KV_EUNSUPPORTED;
+    // the step count of the whole batch is summed in 32 bits
+    const int64_t max_ctx = table_cols * bs;
+    if (bs > (1 << 24) || table_cols > (1 << 24) || batch * ((max_ctx + kStep - 1) / kStep) > 0x7fffffffLL)
+        return INFER_KV_EINVAL;
     return INFER_KV_OK;
+}
+
+struct DecodeCall {
+    const void* q; int64_t q_stride0;
+    const void* k_cache; const void* v_cache;
+    int64_t cache_block_stride, cache_token_stride;
+    const int32_t* block_table; int64_t bt_stride0, table_cols;
+    const int32_t* context_lens;
+    int64_t batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks;
+    float scale;
+};
+
+// Checks every argument of the split phase and fills in the launch shape.
+int check_split(const DecodeCall& c, int64_t split_workgroups, const void* workspace, Launch* L) {
+    if (!c.q || !c.k_cache || !c.v_cache || !c.block_table || !c.context_lens || !workspace) return INFER_KV_EINVAL;
+    int rc = check_shape(c.batch, c.num_q_heads, c.num_kv_heads, c.head_dim, c.block_size, c.num_blocks, c.table_cols);
+    if (rc) return rc;
+    // 16-byte vector loads: every row start must be 16-byte aligned.
+    if (((uintptr_t)c.q | (uintptr_t)c.k_cache | (uintptr_t)c.v_cache | (uintptr_t)workspace) & 15) return INFER_KV_EALIGN;
+    if ((c.q_stride0 | c.cache_block_stride | c.cache_token_stride) & 7) return INFER_KV_EALIGN;
+    if (c.cache_token_stride < c.num_kv_heads * kD || c.cache_block_stride < c.block_size * c.cache_token_stride)
+        return INFER_KV_EINVAL;
+    if (c.batch > 1 && c.bt_stride0 < c.table_cols) return INFER_KV_EINVAL;
+    // lane offsets inside one step are kept in 32 bits
+    if (32 * c.cache_token_stride >= (int64_t)1 << 31) return INFER_KV_EINVAL;
+    return plan_launch(c.num_kv_heads, split_workgroups, L);
+}
+
+int check_out(const void* out, int64_t out_stride0, int64_t num_q_heads) {
+    if (!out || out_stride0 < num_q_heads * kD) return INFER_KV_EINVAL;
+    // 8-byte stores of four outputs
+    if (((uintptr_t)out & 7) || (out_stride0 & 3)) return INFER_KV_EALIGN;
+    return INFER_KV_OK;
+}
+
+// Enqueues the split kernel; `base` is device memory laid out as `ws` (arguments already checked).
+int launch_split(const DecodeCall& c, const Launch& L, const DecodeWorkspace& ws, void* base_v, hipStream_t stream) {
+    DecodeArgs a;
+    a.q = (const uint16_t*)c.q;
+    a.q_stride0 = c.q_stride0;
+    a.k = (const uint16_t*)c.k_cache;
+    a.v = (const uint16_t*)c.v_cache;
+    a.blk_stride = c.cache_block_stride;
+    a.tok_stride = c.cache_token_stride;
+    a.bt = c.block_table;
+    a.bt_stride0 = c.bt_stride0;
+    a.ctx = c.context_lens;
+    const int64_t max_ctx = c.table_cols * c.block_size;
+    a.max_ctx = max_ctx > 0x7fffffffLL ? 0x7fffffff : (int)max_ctx;
+    a.batch = (int)c.batch;
+    a.group = (int)(c.num_q_heads / c.num_kv_heads);
+    a.num_kv_heads = (int)c.num_kv_heads;
+    a.block_size = (int)c.block_size;
+    a.num_blocks = (int)c.num_blocks;
+    a.scale_log2 = c.scale * 1.4426950408889634f;
+    char* base = (char*)base_v;
+    a.header = (int32_t*)(base + ws.header_off);
+    a.seg_first = (int32_t*)(base + ws.seg_first_off);
+    a.seg_last = (int32_t*)(base + ws.seg_last_off);
+    a.rec = (unsigned char*)base + ws.rec_off;
+    a.rec_stride = (int)ws.rec_stride;
+    a.slots_per_head = (int)ws.slots_per_head;
+
+    const size_t lds_bytes = (size_t)L.waves * kLdsPerWave;
+    static bool attr_set[kMaxDevices] = {false};   // the attribute is per device
+    const int dev = current_device();
+    if (!attr_set[dev]) {
+        hipError_t e = hipFuncSetAttribute((const void*)paged_decode_split_kernel,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 8 * kLdsPerWave);
+        if (e != hipSuccess) return (int)e;
+        attr_set[dev] = true;
+    }
+    dim3 grid(L.W, L.grid_y, 1), block(64 * L.waves, 1, 1);
+    hipLaunchKernelGGL(paged_decode_split_kernel, grid, block, lds_bytes, stream, a);
+    return (int)hipGetLastError();
+}
+
+int launch_merge(void* out, int64_t out_stride0, const int32_t* context_lens, int64_t batch, int64_t num_q_heads,
+                 int64_t num_kv_heads, const DecodeWorkspace& ws, const void* base_v, hipStream_t stream) {
+    const char* base = (const char*)base_v;
+    MergeArgs m;
+    m.out = (uint16_t*)out;
+    m.out_stride0 = out_stride0;
+    m.ctx = context_lens;
+    m.group = (int)(num_q_heads / num_kv_heads);
+    m.slots_per_head = (int)ws.slots_per_head;
+    m.seg_first = (const int32_t*)(base + ws.seg_first_off);
+    m.seg_last = (const int32_t*)(base + ws.seg_last_off);
+    m.rec = (const unsigned char*)base + ws.rec_off;
+    m.rec_stride = (int)ws.rec_stride;
+    m.batch = (int)batch;
+    dim3 grid((unsigned)batch, (unsigned)num_q_heads, 1), block(256, 1, 1);
+    hipLaunchKernelGGL(paged_decode_merge_kernel, grid, block, 0, stream, m);
+    return (int)hipGetLastError();
 }
 
 }  // namespace
@@ -673,121 +778,62 @@ size_t infer_paged_decode_workspace_bytes(int64_t max_batch, int64_t num_q_heads
     return ws.total_bytes;
 }
 
-int infer_paged_decode_set_split_workgroups(int workgroups) {
-    int prev = g_split_workgroups;
-    g_split_workgroups = workgroups < 0 ? 0 : workgroups;
-    return prev;
-}
-
 int infer_paged_decode_split_bf16(const void* q, int64_t q_stride0, const void* k_cache, const void* v_cache,
                                   int64_t cache_block_stride, int64_t cache_token_stride,
-                                  const int32_t* block_table, int64_t bt_stride0, const int32_t* context_lens,
-                                  int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
-                                  int64_t block_size, int64_t num_blocks, float scale, void* workspace,
-                                  size_t workspace_bytes, void* stream) {
-    if (!q || !k_cache || !v_cache || !block_table || !context_lens || !workspace) return INFER_KV_EINVAL;
-    int rc = check_shape(batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks);
-    if (rc) return rc;
-    // 16-byte vector loads: every row start must be 16-byte aligned.
-    if (((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)workspace) & 15) return INFER_KV_EALIGN;
-    if ((q_stride0 | cache_block_stride | cache_token_stride) & 7) return INFER_KV_EALIGN;
-    if (cache_token_stride < num_kv_heads * kD || cache_block_stride < block_size * cache_token_stride) return INFER_KV_EINVAL;
-    // lane offsets inside one step are kept in 32 bits
-    if (32 * cache_token_stride >= (int64_t)1 << 31) return INFER_KV_EINVAL;
+                                  const int32_t* block_table, int64_t bt_stride0, int64_t table_cols,
+                                  const int32_t* context_lens, int64_t batch, int64_t num_q_heads,
+                                  int64_t num_kv_heads, int64_t head_dim, int64_t block_size, int64_t num_blocks,
+                                  float scale, int64_t split_workgroups, void* workspace, size_t workspace_bytes,
+                                  void* stream) {
+    const DecodeCall c{q, q_stride0, k_cache, v_cache, cache_block_stride, cache_token_stride, block_table, bt_stride0,
+                       table_cols, context_lens, batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks,
+                       scale};
     Launch L;
-    rc = plan_launch(num_kv_heads, &L);
+    int rc = check_split(c, split_workgroups, workspace, &L);
     if (rc) return rc;
-    const int G = (int)(num_q_heads / num_kv_heads);
-    DecodeWorkspace ws = decode_workspace_layout(batch, G, num_kv_heads);
+    const DecodeWorkspace ws = decode_workspace_layout(batch, num_q_heads / num_kv_heads, num_kv_heads);
     if (ws.total_bytes > workspace_bytes) return INFER_KV_EWORKSPACE;
-
-    DecodeArgs a;
-    a.q = (const uint16_t*)q;
-    a.q_stride0 = q_stride0;
-    a.k = (const uint16_t*)k_cache;
-    a.v = (const uint16_t*)v_cache;
-    a.blk_stride = cache_block_stride;
-    a.tok_stride = cache_token_stride;
-    a.bt = block_table;
-    a.bt_stride0 = bt_stride0;
-    a.ctx = context_lens;
-    a.batch = (int)batch;
-    a.group = G;
-    a.num_kv_heads = (int)num_kv_heads;
-    a.block_size = (int)block_size;
-    a.num_blocks = (int)num_blocks;
-    a.scale_log2 = scale * 1.4426950408889634f;
-    char* base = (char*)workspace;
-    a.header = (int32_t*)(base + ws.header_off);
-    a.seg_first = (int32_t*)(base + ws.seg_first_off);
-    a.seg_last = (int32_t*)(base + ws.seg_last_off);
-    a.rec = (unsigned char*)base + ws.rec_off;
-    a.rec_stride = (int)ws.rec_stride;
-    a.slots_per_head = L.W + (int)batch;
-
-    const size_t lds_bytes = (size_t)L.waves * kLdsPerWave;
-    static bool attr_set[kMaxDevices] = {false};   // the attribute is per device
-    const int dev = current_device();
-    if (!attr_set[dev]) {
-        hipError_t e = hipFuncSetAttribute((const void*)paged_decode_split_kernel,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 8 * kLdsPerWave);
-        if (e != hipSuccess) return (int)e;
-        attr_set[dev] = true;
-    }
-    dim3 grid(L.W, L.grid_y, 1), block(64 * L.waves, 1, 1);
-    hipLaunchKernelGGL(paged_decode_split_kernel, grid, block, lds_bytes, (hipStream_t)stream, a);
-    return (int)hipGetLastError();
+    return launch_split(c, L, ws, workspace, (hipStream_t)stream);
 }
 
 int infer_paged_decode_merge_bf16(void* out, int64_t out_stride0, const int32_t* context_lens, int64_t batch,
                                   int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
                                   const void* workspace, size_t workspace_bytes, void* stream) {
     if (!out || !context_lens || !workspace) return INFER_KV_EINVAL;
-    if (batch <= 0 || num_q_heads <= 0 || num_kv_heads <= 0) return INFER_KV_EINVAL;
+    if (batch <= 0 || batch > (1 << 20) || num_q_heads <= 0 || num_kv_heads <= 0) return INFER_KV_EINVAL;
     if (head_dim != kD) return INFER_KV_EUNSUPPORTED;
     if (num_q_heads % num_kv_heads != 0 || num_q_heads / num_kv_heads > 16) return INFER_KV_EUNSUPPORTED;
-    if (out_stride0 < num_q_heads * kD) return INFER_KV_EINVAL;
-    // 8-byte stores of four outputs; 16-byte loads of the records
-    if (((uintptr_t)out & 7) || (out_stride0 & 3) || ((uintptr_t)workspace & 15)) return INFER_KV_EALIGN;
-    const int G = (int)(num_q_heads / num_kv_heads);
-    DecodeWorkspace ws = decode_workspace_layout(batch, G, num_kv_heads);
-    if (ws.total_bytes > workspace_bytes) return INFER_KV_EWORKSPACE;
-    Launch L;
-    int rc = plan_launch(num_kv_heads, &L);   // same knob -> same split count as the split launch
+    int rc = check_out(out, out_stride0, num_q_heads);
     if (rc) return rc;
-    const char* base = (const char*)workspace;
-    MergeArgs m;
-    m.out = (uint16_t*)out;
-    m.out_stride0 = out_stride0;
-    m.ctx = context_lens;
-    m.group = G;
-    m.split_workgroups = L.W;
-    m.seg_first = (const int32_t*)(base + ws.seg_first_off);
-    m.seg_last = (const int32_t*)(base + ws.seg_last_off);
-    m.rec = (const unsigned char*)base + ws.rec_off;
-    m.rec_stride = (int)ws.rec_stride;
-    m.batch = (int)batch;
-    dim3 grid((unsigned)batch, (unsigned)num_q_heads, 1), block(256, 1, 1);
-    hipLaunchKernelGGL(paged_decode_merge_kernel, grid, block, 0, (hipStream_t)stream, m);
-    return (int)hipGetLastError();
+    if ((uintptr_t)workspace & 15) return INFER_KV_EALIGN;   // 16-byte loads of the records
+    const DecodeWorkspace ws = decode_workspace_layout(batch, num_q_heads / num_kv_heads, num_kv_heads);
+    if (ws.total_bytes > workspace_bytes) return INFER_KV_EWORKSPACE;
+    return launch_merge(out, out_stride0, context_lens, batch, num_q_heads, num_kv_heads, ws, workspace,
+                        (hipStream_t)stream);
 }
 
 int infer_paged_decode_bf16(const void* q, int64_t q_stride0, const void* k_cache, const void* v_cache,
                             int64_t cache_block_stride, int64_t cache_token_stride, void* out,
-                            int64_t out_stride0, const int32_t* block_table, int64_t bt_stride0,
+                            int64_t out_stride0, const int32_t* block_table, int64_t bt_stride0, int64_t table_cols,
                             const int32_t* context_lens, int64_t batch, int64_t num_q_heads,
                             int64_t num_kv_heads, int64_t head_dim, int64_t block_size, int64_t num_blocks,
-                            float scale, void* workspace, size_t workspace_bytes, void* stream) {
-    // what the merge launch would reject is rejected before the split launch is enqueued
-    if (!out || out_stride0 < num_q_heads * kD) return INFER_KV_EINVAL;
-    if (((uintptr_t)out & 7) || (out_stride0 & 3)) return INFER_KV_EALIGN;
-    int rc = infer_paged_decode_split_bf16(q, q_stride0, k_cache, v_cache, cache_block_stride, cache_token_stride,
-                                           block_table, bt_stride0, context_lens, batch, num_q_heads,
-                                           num_kv_heads, head_dim, block_size, num_blocks, scale, workspace,
-                                           workspace_bytes, stream);
+                            float scale, int64_t split_workgroups, void* workspace, size_t workspace_bytes,
+                            void* stream) {
+    const DecodeCall c{q, q_stride0, k_cache, v_cache, cache_block_stride, cache_token_stride, block_table, bt_stride0,
+                       table_cols, context_lens, batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks,
+                       scale};
+    // everything is checked before the first launch is enqueued
+    Launch L;
+    int rc = check_split(c, split_workgroups, workspace, &L);
     if (rc) return rc;
-    return infer_paged_decode_merge_bf16(out, out_stride0, context_lens, batch, num_q_heads, num_kv_heads,
-                                         head_dim, workspace, workspace_bytes, stream);
+    rc = check_out(out, out_stride0, num_q_heads);
+    if (rc) return rc;
+    const DecodeWorkspace ws = decode_workspace_layout(batch, num_q_heads / num_kv_heads, num_kv_heads);
+    if (ws.total_bytes > workspace_bytes) return INFER_KV_EWORKSPACE;
+    rc = launch_split(c, L, ws, workspace, (hipStream_t)stream);
+    if (rc) return rc;
+    return launch_merge(out, out_stride0, context_lens, batch, num_q_heads, num_kv_heads, ws, workspace,
+                        (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -56,6 +56,7 @@ struct PrefillArgs {
     int qblocks_per_wg;     // consecutive query blocks one workgroup covers
     int block_size;
     int num_blocks;
+    int max_sk;             // paged keys: what a block-table row can address (table_cols * block_size)
     float scale_log2;
     int causal;
 };
@@ -123,7 +124,9 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
 
     const int q_beg = a.cu_q[b], q_end = a.cu_q[b + 1];
     const int k_beg = a.cu_k[b], k_end = a.cu_k[b + 1];
-    const int sq = q_end - q_beg, sk = k_end - k_beg;
+    const int sq = q_end - q_beg;
+    int sk = k_end - k_beg;
+    if (a.bt != nullptr && sk > a.max_sk) sk = a.max_sk;   // a corrupt length cannot run the gather past its table row
     // late query blocks see the most keys: hand them out first so the long workgroups start early
     const int wg_q0 = (int)(gridDim.x - 1 - blockIdx.x) * QB * kQBlock;
     if (wg_q0 >= sq) return;
@@ -204,7 +207,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     auto dma16 = [&](const uint16_t* base, uint32_t byte_off, unsigned char* dst) {
         const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)dst;
         __asm__ volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                         :: "v"(byte_off), "s"(base), "s"(lds_addr) : "memory");
+                         :: "v"(byte_off), "s"(base), "s"(lds_addr) : "memory", "m0");
     };
     constexpr int kLoads = (16 + WAVES - 1) / WAVES;
     const int tok_stride = (int)a.tok_stride;     // < 2^24 elements (checked on the host)
@@ -411,7 +414,7 @@ extern "C" int infer_paged_prefill_bf16(const void* q, int64_t q_stride0, const 
                                         int64_t kv_block_stride, int64_t kv_token_stride, int64_t kv_rows,
                                         void* out, int64_t out_stride0, const int32_t* cu_seqlens_q,
                                         const int32_t* cu_seqlens_k, const int32_t* block_table, int64_t bt_stride0,
-                                        int64_t num_seqs, int64_t max_seqlen_q, int64_t num_q_heads,
+                                        int64_t table_cols, int64_t num_seqs, int64_t max_seqlen_q, int64_t num_q_heads,
                                         int64_t num_kv_heads, int64_t head_dim, int64_t block_size,
                                         int64_t num_blocks, float scale, int causal, void* stream) {
     if (!q || !k || !v || !out || !cu_seqlens_q || !cu_seqlens_k) return INFER_KV_EINVAL;
@@ -419,7 +422,11 @@ extern "C" int infer_paged_prefill_bf16(const void* q, int64_t q_stride0, const 
     if (max_seqlen_q == 0) return INFER_KV_OK;
     if (head_dim != kD) return INFER_KV_EUNSUPPORTED;
     if (num_q_heads % num_kv_heads != 0 || num_q_heads / num_kv_heads > 16) return INFER_KV_EUNSUPPORTED;
+    // the row maximum is taken before the scale is applied, which needs a positive scale
+    if (!(scale > 0.f)) return INFER_KV_EINVAL;
     if (block_table && (block_size <= 0 || block_size % kStep != 0 || num_blocks <= 0)) return INFER_KV_EUNSUPPORTED;
+    if (block_table && (table_cols <= 0 || (num_seqs > 1 && bt_stride0 < table_cols) || table_cols * block_size > 0x7fffffffLL))
+        return INFER_KV_EINVAL;
     if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) return INFER_KV_EALIGN;
     if ((q_stride0 | kv_token_stride | out_stride0) & 7) return INFER_KV_EALIGN;
     if (block_table && (kv_block_stride & 7)) return INFER_KV_EALIGN;
@@ -446,6 +453,7 @@ extern "C" int infer_paged_prefill_bf16(const void* q, int64_t q_stride0, const 
     a.bt = block_table; a.bt_stride0 = bt_stride0;
     a.group = G;
     a.block_size = (int)block_size; a.num_blocks = (int)num_blocks;
+    a.max_sk = block_table ? (int)(table_cols * block_size) : 0x7fffffff;
     a.scale_log2 = scale * 1.4426950408889634f;
     a.causal = causal ? 1 : 0;
     hipStream_t st = (hipStream_t)stream;

@@ -1,12 +1,15 @@
 // Streaming probes: what this GPU sustains for a read-only stream and for a plain copy, measured
 // with the same launch shape as the decode kernel (one workgroup of 512 threads per span, 16-byte
-// loads, three batches of eight loads in flight per lane).  Not part of the KV-cache path; bench.py
-// --ceiling uses it to put the kernels' achieved bandwidth next to the practical ceiling of the part.
-// Two copy shapes: a grid-stride loop, and the append kernel's own shape (one wavefront per 4 KiB).
+// loads, three batches of eight loads in flight per lane).  Not part of the KV-cache path and not part
+// of libinfer_kv.so: built as libinfer_kv_probe.so, which only bench.py --ceiling / --counters load, to
+// put the kernels' achieved bandwidth next to the practical ceiling of the part.
+// Copy shapes: a grid-stride loop, the small append kernel's shape (one wavefront per 4 KiB), and the
+// two halves of the KV append on their own (gather the source rows without storing them, scatter
+// rows to their slots without loading any).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include "../../include/infer_kv.h"
+#include "../../include/infer_kv_probe.h"
 
 namespace {
 
@@ -64,9 +67,64 @@ __global__ void __launch_bounds__(256) stream_copy_rows_kernel(const u32x4* __re
     for (int u = 0; u < 4; ++u) __builtin_nontemporal_store(r[u], dst + base + lane + 64 * u);
 }
 
+// Read half of the KV append: every row with a valid slot is loaded (K and V, 2 KiB each), nothing
+// is stored.  One wavefront per row, as the append kernel for few rows.
+__global__ void __launch_bounds__(256) append_read_half_kernel(const u32x4* __restrict__ key, const u32x4* __restrict__ value,
+                                                               const int32_t* __restrict__ slots, int n_rows,
+                                                               int num_slots, uint32_t* sink) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= n_rows) return;
+    const int slot = __builtin_amdgcn_readfirstlane(slots[row]);
+    if (slot < 0 || slot >= num_slots) return;
+    const u32x4* ks = key + (size_t)row * 128;
+    const u32x4* vs = value + (size_t)row * 128;
+    const u32x4 x = __builtin_nontemporal_load(ks + lane) ^ __builtin_nontemporal_load(ks + lane + 64) ^
+                    __builtin_nontemporal_load(vs + lane) ^ __builtin_nontemporal_load(vs + lane + 64);
+    if (fold(x) == 0x9e3779b9u) *sink = 1;   // keeps the loads alive; practically never true
+}
+
+// Write half: every row with a valid slot is stored to its slot in both caches, nothing is loaded.
+__global__ void __launch_bounds__(256) append_write_half_kernel(u32x4* __restrict__ k_cache, u32x4* __restrict__ v_cache,
+                                                                const int32_t* __restrict__ slots, int n_rows,
+                                                                int num_slots) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= n_rows) return;
+    const int slot = __builtin_amdgcn_readfirstlane(slots[row]);
+    if (slot < 0 || slot >= num_slots) return;
+    u32x4* kd = k_cache + (size_t)slot * 128;
+    u32x4* vd = v_cache + (size_t)slot * 128;
+    const u32x4 r = {(uint32_t)row, 1u, 2u, 3u};
+    __builtin_nontemporal_store(r, kd + lane);
+    __builtin_nontemporal_store(r, kd + lane + 64);
+    __builtin_nontemporal_store(r, vd + lane);
+    __builtin_nontemporal_store(r, vd + lane + 64);
+}
+
 }  // namespace
 
 extern "C" {
+
+int infer_kv_probe_append_read_half(const void* key, const void* value, const int32_t* slot_mapping, int64_t n_rows,
+                                    int64_t num_slots, void* sink4, void* stream) {
+    if (!key || !value || !slot_mapping || !sink4 || n_rows <= 0 || n_rows > 0x7fffffffLL || num_slots <= 0 ||
+        num_slots > 0x7fffffffLL || (((uintptr_t)key | (uintptr_t)value) & 15))
+        return INFER_KV_EINVAL;
+    hipLaunchKernelGGL(append_read_half_kernel, dim3((unsigned)((n_rows + 3) / 4)), dim3(256), 0, (hipStream_t)stream,
+                       (const u32x4*)key, (const u32x4*)value, slot_mapping, (int)n_rows, (int)num_slots, (uint32_t*)sink4);
+    return (int)hipGetLastError();
+}
+
+int infer_kv_probe_append_write_half(void* k_cache, void* v_cache, const int32_t* slot_mapping, int64_t n_rows,
+                                     int64_t num_slots, void* stream) {
+    if (!k_cache || !v_cache || !slot_mapping || n_rows <= 0 || n_rows > 0x7fffffffLL || num_slots <= 0 ||
+        num_slots > 0x7fffffffLL || (((uintptr_t)k_cache | (uintptr_t)v_cache) & 15))
+        return INFER_KV_EINVAL;
+    hipLaunchKernelGGL(append_write_half_kernel, dim3((unsigned)((n_rows + 3) / 4)), dim3(256), 0, (hipStream_t)stream,
+                       (u32x4*)k_cache, (u32x4*)v_cache, slot_mapping, (int)n_rows, (int)num_slots);
+    return (int)hipGetLastError();
+}
 
 int infer_kv_probe_read(const void* src, size_t bytes, void* sink4, int workgroups, void* stream) {
     if (!src || !sink4 || bytes < 16 || workgroups <= 0 || ((uintptr_t)src & 15)) return INFER_KV_EINVAL;

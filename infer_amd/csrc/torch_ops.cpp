@@ -27,10 +27,16 @@ void check_bf16_cuda(const at::Tensor& t, const char* name) {
 }
 
 // Split-KV workspace, one per (device, head shape), grown on demand and then reused so that
-// steady-state steps and graph replays do not allocate.
-at::Tensor& decode_workspace(const at::Tensor& like, int64_t batch, int64_t hq, int64_t hkv, int64_t d) {
+// steady-state steps and graph replays do not allocate.  A workspace that a larger batch outgrows
+// stays alive for the life of the process: a HIP graph captured at the smaller batch still points
+// at it, and its replays must keep writing to memory nobody else owns.  The buffer is shared by all
+// calls for the shape, so those calls must be ordered on one stream (the partial results of one call
+// are live until its merge kernel has run); callers that decode the same shape on several streams
+// at once call infer_paged_decode_bf16 with a workspace per stream instead.
+at::Tensor decode_workspace(const at::Tensor& like, int64_t batch, int64_t hq, int64_t hkv, int64_t d) {
     static std::mutex mu;
     static std::unordered_map<std::string, std::pair<int64_t, at::Tensor>> cache;
+    static std::vector<at::Tensor> retired;
     std::lock_guard<std::mutex> g(mu);
     const std::string key = std::to_string(like.get_device()) + ":" + std::to_string(hq) + ":" + std::to_string(hkv) + ":" + std::to_string(d);
     auto& slot = cache[key];
@@ -38,6 +44,7 @@ at::Tensor& decode_workspace(const at::Tensor& like, int64_t batch, int64_t hq, 
         const int64_t cap = std::max<int64_t>(batch, slot.second.defined() ? 2 * slot.first : 64);
         const size_t bytes = infer_paged_decode_workspace_bytes(cap, hq, hkv, d);
         TORCH_CHECK(bytes > 0, "paged decode: unsupported shape (Hq=", hq, ", Hkv=", hkv, ", D=", d, ")");
+        if (slot.second.defined()) retired.push_back(slot.second);
         slot = {cap, at::empty({static_cast<int64_t>(bytes)}, like.options().dtype(at::kByte))};
     }
     return slot.second;
@@ -72,17 +79,18 @@ void paged_attn_decode(const at::Tensor& q, const at::Tensor& k_cache, const at:
     const int64_t b = q.size(0), hq = q.size(1), d = q.size(2), hkv = k_cache.size(2);
     TORCH_CHECK(q.stride(2) == 1 && q.stride(1) == d && out.stride(2) == 1 && out.stride(1) == d, "q/out heads must be contiguous");
     TORCH_CHECK(k_cache.size(3) == d && k_cache.stride(3) == 1 && k_cache.stride(2) == d, "cache heads must be contiguous");
-    TORCH_CHECK(block_table.is_cuda() && block_table.scalar_type() == at::kInt && block_table.size(0) == b && block_table.stride(1) == 1,
-                "block_table must be int32 [B, MB]");
+    TORCH_CHECK(block_table.is_cuda() && block_table.scalar_type() == at::kInt && block_table.dim() == 2 && block_table.size(0) == b && block_table.size(1) >= 1 && block_table.stride(1) == 1,
+                "block_table must be int32 [B, MB] with MB >= 1");
     TORCH_CHECK(context_lens.is_cuda() && context_lens.scalar_type() == at::kInt && context_lens.numel() == b && context_lens.is_contiguous(),
                 "context_lens must be int32 [B]");
     if (b == 0) return;
     DeviceGuard guard(q.device());
-    at::Tensor& ws = decode_workspace(q, b, hq, hkv, d);
+    at::Tensor ws = decode_workspace(q, b, hq, hkv, d);
     check_rc(infer_paged_decode_bf16(q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), k_cache.stride(0),
                                      k_cache.stride(1), out.data_ptr(), out.stride(0), block_table.data_ptr<int>(),
-                                     block_table.stride(0), context_lens.data_ptr<int>(), b, hq, hkv, d, k_cache.size(1),
-                                     k_cache.size(0), static_cast<float>(scale), ws.data_ptr(), ws.numel(), current_stream()),
+                                     block_table.stride(0), block_table.size(1), context_lens.data_ptr<int>(), b, hq, hkv, d,
+                                     k_cache.size(1), k_cache.size(0), static_cast<float>(scale), /*split_workgroups=*/0,
+                                     ws.data_ptr(), ws.numel(), current_stream()),
              "paged_attn_decode");
 }
 
@@ -113,14 +121,14 @@ void paged_attn_prefill(const at::Tensor& q, const at::Tensor& k, const at::Tens
         TORCH_CHECK(bt.is_cuda() && bt.scalar_type() == at::kInt && bt.size(0) == nseq && bt.stride(1) == 1, "block_table must be int32 [nseq, MB]");
         rc = infer_paged_prefill_bf16(q.data_ptr(), q.stride(0), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1),
                                       k.size(0) * k.size(1), out.data_ptr(), out.stride(0), cu_seqlens_q.data_ptr<int>(),
-                                      cu_seqlens_k.data_ptr<int>(), bt.data_ptr<int>(), bt.stride(0), nseq, max_seqlen_q, hq,
+                                      cu_seqlens_k.data_ptr<int>(), bt.data_ptr<int>(), bt.stride(0), bt.size(1), nseq, max_seqlen_q, hq,
                                       k.size(2), d, k.size(1), k.size(0), static_cast<float>(scale), causal, current_stream());
     } else {
         TORCH_CHECK(k.dim() == 3 && k.sizes() == v.sizes() && k.strides() == v.strides() && k.size(2) == d &&
                     k.stride(2) == 1 && k.stride(1) == d, "packed k/v must be [T, Hkv, D]");
         rc = infer_paged_prefill_bf16(q.data_ptr(), q.stride(0), k.data_ptr(), v.data_ptr(), 0, k.stride(0), k.size(0),
                                       out.data_ptr(), out.stride(0), cu_seqlens_q.data_ptr<int>(), cu_seqlens_k.data_ptr<int>(),
-                                      nullptr, 0, nseq, max_seqlen_q, hq, k.size(1), d, 0, 0, static_cast<float>(scale),
+                                      nullptr, 0, 0, nseq, max_seqlen_q, hq, k.size(1), d, 0, 0, static_cast<float>(scale),
                                       causal, current_stream());
     }
     check_rc(rc, "paged_attn_prefill");

@@ -119,14 +119,19 @@ def _decode_args(q3, k_cache, v_cache, cache_seqlens, block_table):
     assert dk == d and q3.stride(2) == 1 and q3.stride(1) == d
     assert k_cache.stride(3) == 1 and k_cache.stride(2) == d
     assert cache_seqlens.numel() == b and cache_seqlens.is_contiguous()
-    assert block_table.shape[0] == b and block_table.stride(1) == 1
+    assert block_table.dim() == 2 and block_table.shape[0] == b and block_table.shape[1] >= 1
+    assert block_table.stride(1) == 1
     _require_gpu(q3, k_cache, v_cache, cache_seqlens, block_table)
     return b, hq, d, nblk, bs, hkv
 
 
 def paged_attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
-                      context_lens: torch.Tensor, scale: float, out: torch.Tensor, workspace=None) -> None:
-    """Out-parameter form: ``q``/``out`` are ``[B, Hq, D]``."""
+                      context_lens: torch.Tensor, scale: float, out: torch.Tensor, workspace=None,
+                      split_workgroups: int = 0) -> None:
+    """Out-parameter form: ``q``/``out`` are ``[B, Hq, D]``.  ``split_workgroups`` = workgroups along
+    the KV-split axis of this call (0: the library's choice for the device).  The default workspace is
+    shared by every call for the shape on the device, so such calls must be ordered on one stream;
+    pass a ``workspace`` of its own to a call that runs on another stream."""
     b, hq, d, nblk, bs, hkv = _decode_args(q, k_cache, v_cache, context_lens, block_table)
     assert out.shape == q.shape and out.dtype == torch.bfloat16 and out.stride(2) == 1 and out.stride(1) == d
     if workspace is None:
@@ -134,18 +139,21 @@ def paged_attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     lib = _lib.load()
     rc = lib.infer_paged_decode_bf16(
         q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), k_cache.stride(0), k_cache.stride(1),
-        out.data_ptr(), out.stride(0), block_table.data_ptr(), block_table.stride(0), context_lens.data_ptr(),
-        b, hq, hkv, d, bs, nblk, float(scale), workspace.data_ptr(), workspace.numel(), _stream_ptr(q))
+        out.data_ptr(), out.stride(0), block_table.data_ptr(), block_table.stride(0), block_table.shape[1],
+        context_lens.data_ptr(), b, hq, hkv, d, bs, nblk, float(scale), int(split_workgroups),
+        workspace.data_ptr(), workspace.numel(), _stream_ptr(q))
     _lib.check(rc, "paged_attn_decode")
 
 
-def paged_attn_decode_split(q, k_cache, v_cache, block_table, context_lens, scale, workspace) -> None:
+def paged_attn_decode_split(q, k_cache, v_cache, block_table, context_lens, scale, workspace,
+                            split_workgroups: int = 0) -> None:
     """Bandwidth-bound phase alone (partials stay in ``workspace``); for profiling."""
     b, hq, d, nblk, bs, hkv = _decode_args(q, k_cache, v_cache, context_lens, block_table)
     rc = _lib.load().infer_paged_decode_split_bf16(
         q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), k_cache.stride(0), k_cache.stride(1),
-        block_table.data_ptr(), block_table.stride(0), context_lens.data_ptr(),
-        b, hq, hkv, d, bs, nblk, float(scale), workspace.data_ptr(), workspace.numel(), _stream_ptr(q))
+        block_table.data_ptr(), block_table.stride(0), block_table.shape[1], context_lens.data_ptr(),
+        b, hq, hkv, d, bs, nblk, float(scale), int(split_workgroups), workspace.data_ptr(), workspace.numel(),
+        _stream_ptr(q))
     _lib.check(rc, "paged_attn_decode_split")
 
 
@@ -208,16 +216,16 @@ def flash_attn_varlen_func(q, k, v, *, max_seqlen_q, cu_seqlens_q, max_seqlen_k,
         assert block_table.dtype == torch.int32 and block_table.shape[0] == nseq and block_table.stride(1) == 1
         _require_gpu(block_table)
         blk_stride, tok_stride, rows = k.stride(0), k.stride(1), nblk * bs
-        bt_ptr, bt_stride = block_table.data_ptr(), block_table.stride(0)
+        bt_ptr, bt_stride, bt_cols = block_table.data_ptr(), block_table.stride(0), block_table.shape[1]
     else:
         assert k.dim() == 3 and k.shape == v.shape and k.stride() == v.stride()
         rows, hkv, dk = k.shape
         assert dk == d and k.stride(2) == 1 and k.stride(1) == d
         blk_stride, tok_stride, bs, nblk = 0, k.stride(0), 0, 0
-        bt_ptr, bt_stride = None, 0
+        bt_ptr, bt_stride, bt_cols = None, 0, 0
     rc = _lib.load().infer_paged_prefill_bf16(
         q.data_ptr(), q.stride(0), k.data_ptr(), v.data_ptr(), blk_stride, tok_stride, rows,
-        out.data_ptr(), out.stride(0), cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), bt_ptr, bt_stride,
+        out.data_ptr(), out.stride(0), cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), bt_ptr, bt_stride, bt_cols,
         nseq, int(max_seqlen_q), hq, hkv, d, bs, nblk, float(softmax_scale), int(bool(causal)), _stream_ptr(q))
     _lib.check(rc, "flash_attn_varlen_func")
     return out
@@ -455,7 +463,3 @@ def linear(x: torch.Tensor, weight: torch.Tensor, defer: bool = False):
         return torch.nn.functional.linear(x, weight)
     # ``defer``: the caller hands the result straight to ``rms_norm``, which adds the partial sums itself
     return skinny_linear_deferred(x, weight) if defer else skinny_linear(x, weight)
-
-
-def set_split_workgroups(n: int) -> int:
-    return _lib.load().infer_paged_decode_set_split_workgroups(int(n))

@@ -55,7 +55,11 @@ class QwenAttention(nn.Module):
         context = get_context()
         k_cache, v_cache, bound = self._caches(q.device)
         slots = context.slot_mapping
-        if not bound or slots is None or slots.numel() != q.shape[0]:
+        if bound:
+            # with a cache bound every token must come with its slot, as the reference's store_kvcache
+            # asserts (infer/ops/attention.py:44): a metadata bug must not silently skip the append
+            assert slots is not None and slots.numel() == q.shape[0], "slot_mapping must hold one slot per token"
+        else:
             slots = torch.full((q.shape[0],), -1, dtype=torch.int32, device=q.device)
         # keys are read back from the packed rows only by a prefill without a cached prefix
         keys_from_rows = context.is_prefill and context.block_tables is None

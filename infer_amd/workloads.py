@@ -3,14 +3,30 @@
 The shapes are the ones the decode step of ``infer/engine/model_runner.py:110-126`` hands to
 ``infer/ops/attention.py:96-122``: new K/V rows ``[N, Hkv, D]``, caches ``[nblk, bs, Hkv, D]``,
 ``slot_mapping [N]`` int32, ``block_table [B, MB]`` int32 padded with -1, ``context_lens [B]``
-int32 (lengths include the token appended this step).  Everything is bf16 and drawn from a
-``torch.Generator`` so the same seed gives the same tensors on the CPU and on the GPU box.
+int32 (lengths include the token appended this step).  Everything is bf16 and drawn from a CPU
+``torch.Generator``, then moved to the requested device, so the same seed gives the same bits on the
+CPU and on the GPU box; ``checksums`` hashes them (``tests/golden/workload_checksums.json`` holds the
+values of the named configurations).  ``device_fill=True`` draws the cache contents on the device
+instead: faster for the multi-gigabyte pools of a bandwidth sweep, but reproducible only per device,
+so parity tests never use it.
 """
 from __future__ import annotations
 
+import hashlib
 from dataclasses import dataclass, field
 
 import torch
+
+
+def checksums(wl) -> dict:
+    """SHA-256 of the bytes of every tensor of a workload (on the host, C order), by field name."""
+    out = {}
+    for name, v in wl.__dict__.items():
+        if isinstance(v, torch.Tensor):
+            t = v.detach().cpu().contiguous()
+            raw = t.view(torch.uint8) if t.numel() else t
+            out[name] = hashlib.sha256(raw.numpy().tobytes() if t.numel() else b"").hexdigest()
+    return out
 
 
 @dataclass
@@ -74,8 +90,17 @@ def _tables(lengths, bs, nblk, gen):
     return tables, torch.tensor(padded, dtype=torch.int32)
 
 
+def _draw_caches(shape, dgen, device, device_fill):
+    if device_fill and str(device) != "cpu":
+        g = torch.Generator(device=device).manual_seed(dgen.initial_seed())
+        return (torch.randn(shape, generator=g, device=device, dtype=torch.bfloat16),
+                torch.randn(shape, generator=g, device=device, dtype=torch.bfloat16))
+    return (torch.randn(shape, generator=dgen, dtype=torch.bfloat16),
+            torch.randn(shape, generator=dgen, dtype=torch.bfloat16))
+
+
 def make_decode_workload(name, lengths, hq, hkv, d=128, bs=256, nblk=None, seed=0, q_scale=1.0,
-                         pool_factor=1.2, device="cpu") -> DecodeWorkload:
+                         pool_factor=1.2, device="cpu", device_fill=False) -> DecodeWorkload:
     """Build one decode step.  ``lengths`` include the token appended this step (so >= 1)."""
     gen = torch.Generator(device="cpu").manual_seed(seed)
     need = sum((n + bs - 1) // bs for n in lengths)
@@ -83,21 +108,19 @@ def make_decode_workload(name, lengths, hq, hkv, d=128, bs=256, nblk=None, seed=
         nblk = max(int(-(-need * pool_factor // 1)), need)
     tables, block_table = _tables(lengths, bs, nblk, gen)
     b = len(lengths)
-    dgen = torch.Generator(device=device).manual_seed(seed + 1)
-    shape = (nblk, bs, hkv, d)
-    k_cache = torch.randn(shape, generator=dgen, device=device, dtype=torch.bfloat16)
-    v_cache = torch.randn(shape, generator=dgen, device=device, dtype=torch.bfloat16)
-    q = (torch.randn((b, hq, d), generator=dgen, device=device, dtype=torch.float32) * q_scale).to(torch.bfloat16)
-    k_new = torch.randn((b, hkv, d), generator=dgen, device=device, dtype=torch.float32).to(torch.bfloat16)
-    v_new = torch.randn((b, hkv, d), generator=dgen, device=device, dtype=torch.float32).to(torch.bfloat16)
+    dgen = torch.Generator(device="cpu").manual_seed(seed + 1)
+    k_cache, v_cache = _draw_caches((nblk, bs, hkv, d), dgen, device, device_fill)
+    q = (torch.randn((b, hq, d), generator=dgen, dtype=torch.float32) * q_scale).to(torch.bfloat16)
+    k_new = torch.randn((b, hkv, d), generator=dgen, dtype=torch.float32).to(torch.bfloat16)
+    v_new = torch.randn((b, hkv, d), generator=dgen, dtype=torch.float32).to(torch.bfloat16)
     slots = [t[-1] * bs + (n - 1) % bs for n, t in zip(lengths, tables)]
     return DecodeWorkload(
         name=name, num_q_heads=hq, num_kv_heads=hkv, head_dim=d, block_size=bs, scale=d ** -0.5,
         q=q, k_new=k_new, v_new=v_new, k_cache=k_cache, v_cache=v_cache,
-        slot_mapping=torch.tensor(slots, dtype=torch.int32).to(device),
-        block_table=block_table.to(device),
-        context_lens=torch.tensor(lengths, dtype=torch.int32).to(device),
-        lengths=list(lengths))
+        slot_mapping=torch.tensor(slots, dtype=torch.int32),
+        block_table=block_table,
+        context_lens=torch.tensor(lengths, dtype=torch.int32),
+        lengths=list(lengths)).to(device)
 
 
 def cfg1(device="cpu") -> DecodeWorkload:
@@ -111,18 +134,18 @@ def cfg2_lengths(batch=64, lo=512, hi=4096, seed=0):
     return torch.randint(lo, hi + 1, (batch,), generator=gen).tolist()
 
 
-def cfg2(device="cpu", batch=64) -> DecodeWorkload:
+def cfg2(device="cpu", batch=64, device_fill=False) -> DecodeWorkload:
     """Qwen3-8B-shaped decode step: 32/8 heads, batch 64, lengths U[512, 4096], pool 1.2x need,
     Q scaled by 1/sqrt(128)."""
     return make_decode_workload("cfg2-qwen3-8b-b64", cfg2_lengths(batch), 32, 8, seed=0,
-                                q_scale=128 ** -0.5, device=device)
+                                q_scale=128 ** -0.5, device=device, device_fill=device_fill)
 
 
-def cfg4(device="cpu", batch=8, ctx=32768, nblk=2048) -> DecodeWorkload:
+def cfg4(device="cpu", batch=8, ctx=32768, nblk=2048, device_fill=False) -> DecodeWorkload:
     """Qwen3-32B-shaped long-context decode: 64/8 heads, batch 8 x 32768 tokens, tables fully
     fragmented over a 2048-block pool."""
     return make_decode_workload("cfg4-qwen3-32b-b8-ctx32k", [ctx] * batch, 64, 8, nblk=nblk, seed=0,
-                                device=device)
+                                device=device, device_fill=device_fill)
 
 
 @dataclass
@@ -186,22 +209,19 @@ def make_prefill_workload(name, lengths, cached, hq, hkv, d=128, bs=256, seed=0,
     row_of_query = torch.nonzero(~is_pad).flatten()
     slot_mapping = torch.full((n_rows,), -1, dtype=torch.int32)
     slot_mapping[row_of_query] = torch.tensor(slots, dtype=torch.int32)
-    dgen = torch.Generator(device=device).manual_seed(seed + 1)
-    shape = (nblk, bs, hkv, d)
-    k_cache = torch.randn(shape, generator=dgen, device=device, dtype=torch.bfloat16)
-    v_cache = torch.randn(shape, generator=dgen, device=device, dtype=torch.bfloat16)
-    q = torch.randn((tq, hq, d), generator=dgen, device=device, dtype=torch.float32).to(torch.bfloat16)
-    k_new = torch.randn((n_rows, hkv, d), generator=dgen, device=device, dtype=torch.float32).to(torch.bfloat16)
-    v_new = torch.randn((n_rows, hkv, d), generator=dgen, device=device, dtype=torch.float32).to(torch.bfloat16)
+    dgen = torch.Generator(device="cpu").manual_seed(seed + 1)
+    k_cache, v_cache = _draw_caches((nblk, bs, hkv, d), dgen, device, False)
+    q = torch.randn((tq, hq, d), generator=dgen, dtype=torch.float32).to(torch.bfloat16)
+    k_new = torch.randn((n_rows, hkv, d), generator=dgen, dtype=torch.float32).to(torch.bfloat16)
+    v_new = torch.randn((n_rows, hkv, d), generator=dgen, dtype=torch.float32).to(torch.bfloat16)
     return PrefillWorkload(
         name=name, num_q_heads=hq, num_kv_heads=hkv, head_dim=d, block_size=bs, scale=d ** -0.5,
         q=q, k_new=k_new, v_new=v_new, k_cache=k_cache, v_cache=v_cache,
-        slot_mapping=slot_mapping.to(device), row_of_query=row_of_query.to(device),
-        block_table=block_table.to(device),
-        cu_seqlens_q=torch.tensor(cu_q, dtype=torch.int32).to(device),
-        cu_seqlens_k=torch.tensor(cu_k, dtype=torch.int32).to(device),
+        slot_mapping=slot_mapping, row_of_query=row_of_query, block_table=block_table,
+        cu_seqlens_q=torch.tensor(cu_q, dtype=torch.int32),
+        cu_seqlens_k=torch.tensor(cu_k, dtype=torch.int32),
         max_seqlen_q=max(n - c for n, c in zip(lengths, cached)), max_seqlen_k=max(lengths),
-        lengths=list(lengths), cached=list(cached))
+        lengths=list(lengths), cached=list(cached)).to(device)
 
 
 def cfg3(device="cpu", nseq=16, lo=64, hi=2048, seed=0, hq=32, hkv=8) -> PrefillWorkload:

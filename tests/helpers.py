@@ -25,3 +25,16 @@ def oracle_decode(wl, k_cache=None, v_cache=None) -> np.ndarray:
 # bf16 attention output against the fp32 CPU oracle: the tolerance the reference uses for its
 # own attention test (test/op.py:283, atol=2e-2) and the bar set for this path.
 ATTN_ATOL = 2e-2
+
+
+def assert_seeded_inputs(wl, name):
+    """The tensors of a named configuration are the ones its seed draws on the CPU: their SHA-256
+    equals tests/golden/workload_checksums.json (written by tests/golden/make_workload_checksums.py)."""
+    import json
+    import os
+    from infer_amd import workloads
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "workload_checksums.json")
+    want = json.load(open(path))[name]
+    assert list(wl.lengths) == want["lengths"]
+    got = workloads.checksums(wl)
+    assert got == want["sha256"], f"{name}: inputs differ from the committed seeds' checksums"

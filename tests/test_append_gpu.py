@@ -5,7 +5,7 @@ import torch
 
 from infer_amd import ops, workloads
 from oracle import paged_ref
-from tests.helpers import bits
+from tests.helpers import assert_seeded_inputs, bits
 
 pytestmark = pytest.mark.gpu
 
@@ -16,7 +16,9 @@ def run_both(key, value, k_cache, v_cache, slots):
     ops.store_kvcache(key, value, kc, vc, slots)
     torch.cuda.synchronize()
     ek, ev = bits(k_cache).copy(), bits(v_cache).copy()
-    paged_ref.append_ref(bits(key), bits(value), ek, ev, slots.cpu().numpy())
+    slots_host = slots.cpu().numpy()
+    if int(slots_host.max(initial=-1)) < ek.shape[0] * ek.shape[1]:      # the oracle has no notion of a slot past the end
+        paged_ref.append_ref(bits(key), bits(value), ek, ev, slots_host)
     return bits(kc), bits(vc), ek, ev
 
 
@@ -31,7 +33,9 @@ def test_cfg1_decode_rows(gpu):
 
 
 def test_cfg3_prefill_rows_with_padding(gpu):
-    wl = workloads.cfg3().to(gpu)
+    wl = workloads.cfg3()
+    assert_seeded_inputs(wl, "cfg3")
+    wl = wl.to(gpu)
     assert int((wl.slot_mapping < 0).sum()) > 0
     gk, gv, ek, ev = run_both(wl.k_new, wl.v_new, wl.k_cache, wl.v_cache, wl.slot_mapping)
     assert np.array_equal(gk, ek) and np.array_equal(gv, ev)
@@ -63,6 +67,33 @@ def test_row_widths(gpu, hkv, d):
     slots = torch.randperm(nblk * bs, generator=g)[:n].to(torch.int32)
     slots[::7] = -1
     gk, gv, ek, ev = run_both(key, val, kc, vc, slots.to(gpu))
+    assert np.array_equal(gk, ek) and np.array_equal(gv, ev)
+
+
+@pytest.mark.parametrize("hkv,d,n", [(8, 128, 3073), (8, 128, 20011), (4, 128, 40000), (16, 128, 9001), (8, 64, 5000),
+                                     (3, 40, 5000)])
+def test_many_rows_take_the_ring_shape(gpu, hkv, d, n):
+    """Above 3072 rows the append runs as a fixed grid of wavefronts that each keep a ring of rows in
+    registers.  Covers: the first row count of that shape, counts that make every wavefront go round
+    its ring more than once (20,011 rows of 2 KiB; 40,000 of 1 KiB; 9,001 of 4 KiB), a width the ring
+    is not built for (falls back to one wavefront per row), strided rows out of a fused qkv
+    projection, padding and out-of-range slots in between."""
+    g = torch.Generator(device="cpu").manual_seed(hkv * 977 + d + n)
+    width = hkv * d
+    nblk = (n + 255) // 256 + 3
+    qkv = torch.randn((n, 3 * width + 16), generator=g).to(torch.bfloat16).to(gpu)
+    key, val = qkv[:, 8:8 + width].view(n, hkv, d), qkv[:, 8 + width:8 + 2 * width].view(n, hkv, d)
+    assert not key.is_contiguous()
+    kc = torch.randn((nblk, 256, hkv, d), generator=g).to(torch.bfloat16).to(gpu)
+    vc = torch.randn((nblk, 256, hkv, d), generator=g).to(torch.bfloat16).to(gpu)
+    slots = torch.randperm(nblk * 256, generator=g)[:n].to(torch.int32)
+    slots[::13] = -1
+    skipped = slots.clone()
+    slots[5::101] = nblk * 256 + 7          # past the end of the cache: skipped like a padding row
+    skipped[5::101] = -1                    # (the oracle knows only the padding value)
+    gk, gv, _, _ = run_both(key, val, kc, vc, slots.to(gpu))
+    ek, ev = bits(kc).copy(), bits(vc).copy()
+    paged_ref.append_ref(bits(key), bits(val), ek, ev, skipped.numpy())
     assert np.array_equal(gk, ek) and np.array_equal(gv, ev)
 
 

@@ -10,14 +10,25 @@ from infer_amd import _lib
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_functions():
-    names = []
-    for fn in sorted(os.listdir(os.path.join(ROOT, "include"))):
-        if fn.endswith(".h"):
-            text = open(os.path.join(ROOT, "include", fn)).read()
-            text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-            names += re.findall(r"\b(infer_[a-z0-9_]+)\s*\(", text)
-    return sorted(set(names))
+def declared_functions(header="infer_kv.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(infer_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_header_belongs_to_a_library():
+    assert sorted(fn for fn in os.listdir(os.path.join(ROOT, "include")) if fn.endswith(".h")) == \
+        ["infer_kv.h", "infer_kv_probe.h"]
+
+
+def test_probe_library_exports_what_its_header_declares():
+    """The measurement kernels live in a library of their own that only bench.py loads."""
+    probe = ctypes.CDLL(os.path.join(ROOT, "infer_amd", "libinfer_kv_probe.so"))
+    names = declared_functions("infer_kv_probe.h")
+    assert len(names) == 6
+    for name in names:
+        assert hasattr(probe, name), f"{name} declared in infer_kv_probe.h but not exported"
+        assert not hasattr(_lib.load(), name), f"{name} must not be part of the product library"
 
 
 def test_header_declares_the_expected_entry_points():
@@ -37,7 +48,7 @@ def test_library_exports_every_declared_symbol_and_binding_covers_it():
 
 def test_host_only_entry_points():
     lib = _lib.load()
-    assert lib.infer_kv_version() == b"0.1"
+    assert lib.infer_kv_version() == b"0.2"
     assert b"workspace" in lib.infer_kv_strerror(-3)
     assert lib.infer_paged_decode_workspace_bytes(64, 32, 8, 128) > 0
     assert lib.infer_paged_decode_workspace_bytes(64, 32, 8, 64) == 0        # head_dim not built
@@ -56,13 +67,27 @@ def test_argument_errors_are_reported_before_anything_is_launched():
     p16 = (p + 15) & ~15
     assert lib.infer_kv_append_bf16(p16, 1024, p16, 1024, p16, p16, p16, 4, 1020, 256, None) == -2   # dkv % 8
     assert lib.infer_kv_append_bf16(p16 + 2, 1024, p16, 1024, p16, p16, p16, 4, 1024, 256, None) == -2
-    assert lib.infer_paged_decode_bf16(None, 0, None, None, 0, 0, None, 0, None, 0, None,
-                                       1, 32, 8, 128, 256, 4, 1.0, None, 0, None) == -1
+    assert lib.infer_paged_decode_bf16(None, 0, None, None, 0, 0, None, 0, None, 0, 1, None,
+                                       1, 32, 8, 128, 256, 4, 1.0, 0, None, 0, None) == -1
     # the combined decode call rejects what its second launch would reject before the first is enqueued
-    assert lib.infer_paged_decode_bf16(p16, 4096, p16, p16, 262144, 1024, p16 + 2, 4096, p16, 1, p16,
-                                       1, 32, 8, 128, 256, 4, 1.0, p16, 1 << 30, None) == -2    # out not 8-byte aligned
-    assert lib.infer_paged_decode_bf16(p16, 4096, p16, p16, 262144, 1024, p16, 4095, p16, 1, p16,
-                                       1, 32, 8, 128, 256, 4, 1.0, p16, 1 << 30, None) == -1    # out rows overlap
+    assert lib.infer_paged_decode_bf16(p16, 4096, p16, p16, 262144, 1024, p16 + 2, 4096, p16, 1, 1, p16,
+                                       1, 32, 8, 128, 256, 4, 1.0, 0, p16, 1 << 30, None) == -2  # out not 8-byte aligned
+    assert lib.infer_paged_decode_bf16(p16, 4096, p16, p16, 262144, 1024, p16, 4095, p16, 1, 1, p16,
+                                       1, 32, 8, 128, 256, 4, 1.0, 0, p16, 1 << 30, None) == -1  # out rows overlap
+    # a block table without columns, a row stride shorter than the row, a negative split count, and a
+    # batch whose step count would not fit 32 bits
+    assert lib.infer_paged_decode_bf16(p16, 4096, p16, p16, 262144, 1024, p16, 4096, p16, 1, 0, p16,
+                                       1, 32, 8, 128, 256, 4, 1.0, 0, p16, 1 << 30, None) == -1
+    assert lib.infer_paged_decode_bf16(p16, 4096, p16, p16, 262144, 1024, p16, 4096, p16, 3, 4, p16,
+                                       2, 32, 8, 128, 256, 4, 1.0, 0, p16, 1 << 30, None) == -1
+    assert lib.infer_paged_decode_bf16(p16, 4096, p16, p16, 262144, 1024, p16, 4096, p16, 4, 4, p16,
+                                       2, 32, 8, 128, 256, 4, 1.0, -1, p16, 1 << 30, None) == -1
+    assert lib.infer_paged_decode_bf16(p16, 4096, p16, p16, 262144, 1024, p16, 4096, p16, 1 << 23, 1 << 23, p16,
+                                       1 << 10, 32, 8, 128, 256, 4, 1.0, 0, p16, 1 << 40, None) == -1
+    # prefill: the scale must be positive (the row maximum is taken before scaling)
+    for bad_scale in (0.0, -0.1, float("nan")):
+        assert lib.infer_paged_prefill_bf16(p16, 4096, p16, p16, 262144, 1024, 1024, p16, 4096, p16, p16, p16, 4, 4,
+                                            1, 16, 32, 8, 128, 256, 4, bad_scale, 1, None) == -1
     assert lib.infer_paged_decode_merge_bf16(p16 + 4, 4096, p16, 1, 32, 8, 128, p16, 1 << 30, None) == -2
     with pytest.raises(RuntimeError, match="workspace too small"):
         _lib.check(-3, "x")

@@ -6,23 +6,22 @@ import pytest
 import torch
 
 from infer_amd import ops, workloads
-from tests.helpers import ATTN_ATOL, bits, f32, oracle_decode
+from tests.helpers import ATTN_ATOL, assert_seeded_inputs, bits, f32, oracle_decode
 
 pytestmark = pytest.mark.gpu
 
 
 def gpu_decode(wl, splits=None):
-    if splits is not None:
-        prev = ops.set_split_workgroups(splits)
-    try:
+    if splits is None:
         out = ops.flash_attn_with_kvcache(wl.q.unsqueeze(1), wl.k_cache, wl.v_cache,
                                           cache_seqlens=wl.context_lens, block_table=wl.block_table,
-                                          softmax_scale=wl.scale, causal=True)
-        torch.cuda.synchronize()
-    finally:
-        if splits is not None:
-            ops.set_split_workgroups(prev)
-    return out[:, 0]
+                                          softmax_scale=wl.scale, causal=True)[:, 0]
+    else:   # the split count is an argument of the call; the library keeps no setting
+        out = torch.empty_like(wl.q)
+        ops.paged_attn_decode(wl.q, wl.k_cache, wl.v_cache, wl.block_table, wl.context_lens, wl.scale, out,
+                              split_workgroups=splits)
+    torch.cuda.synchronize()
+    return out
 
 
 def check(wl, splits=None, atol=ATTN_ATOL):
@@ -222,12 +221,9 @@ def test_span_count_reported_in_the_workspace_header(gpu, w):
     for lens in ([4000, 77, 1300, 2048, 31, 900] * 4, [40, 33, 1], workloads.cfg2_lengths(64)):
         wl = workloads.make_decode_workload("hdr", lens, 32, 8, seed=5).to(gpu)
         ws = ops.decode_workspace(gpu, len(lens), 32, 8, 128)
-        prev = ops.set_split_workgroups(w)
-        try:
-            ops.paged_attn_decode_split(wl.q, wl.k_cache, wl.v_cache, wl.block_table, wl.context_lens, wl.scale, ws)
-            torch.cuda.synchronize()
-        finally:
-            ops.set_split_workgroups(prev)
+        ops.paged_attn_decode_split(wl.q, wl.k_cache, wl.v_cache, wl.block_table, wl.context_lens, wl.scale, ws,
+                                    split_workgroups=w)
+        torch.cuda.synchronize()
         spans, total = (int(v) for v in ws[:8].view(torch.int32)[:2].tolist())
         assert total == sum((n + 31) // 32 for n in lens)
         if total <= w:
@@ -240,13 +236,17 @@ def test_span_count_reported_in_the_workspace_header(gpu, w):
 
 
 def test_cfg2_full_size(gpu):
-    wl = workloads.cfg2(device=gpu)
+    wl = workloads.cfg2()                 # drawn on the CPU from the seed, the bits the checksums name
+    assert_seeded_inputs(wl, "cfg2")
+    wl = wl.to(gpu)
     err = check(wl)
     print("cfg2 max abs err", err)
 
 
 def test_cfg4_long_context(gpu):
-    wl = workloads.cfg4(device=gpu)
+    wl = workloads.cfg4()
+    assert_seeded_inputs(wl, "cfg4")
+    wl = wl.to(gpu)
     err = check(wl)
     print("cfg4 max abs err", err)
 
@@ -271,3 +271,66 @@ def test_errors_are_loud(gpu):
     kc = torch.zeros((2, 256, 8, 64), dtype=torch.bfloat16, device=gpu)
     with pytest.raises(RuntimeError):
         ops.flash_attn_with_kvcache(q64, kc, kc, cache_seqlens=wl.context_lens, block_table=wl.block_table)
+
+
+def test_two_streams_with_different_split_counts(gpu):
+    """The split count is per call and the library holds no launch state: two decode calls with
+    different counts, each with its own workspace, run concurrently on two streams and both match
+    the oracle; the same two calls run one after the other give the same bits."""
+    wa = workloads.make_decode_workload("s0", [1500, 700, 2300, 90] * 4, 32, 8, seed=11).to(gpu)
+    wb = workloads.make_decode_workload("s1", [3100, 33, 512] * 3, 32, 8, seed=12).to(gpu)
+    lib_bytes = ops._lib.load().infer_paged_decode_workspace_bytes
+    ws_a = torch.empty(lib_bytes(16, 32, 8, 128), dtype=torch.uint8, device=gpu)
+    ws_b = torch.empty(lib_bytes(9, 32, 8, 128), dtype=torch.uint8, device=gpu)
+    serial = []
+    for wl, ws, w in ((wa, ws_a, 37), (wb, ws_b, 256)):
+        out = torch.empty_like(wl.q)
+        ops.paged_attn_decode(wl.q, wl.k_cache, wl.v_cache, wl.block_table, wl.context_lens, wl.scale, out, ws,
+                              split_workgroups=w)
+        serial.append(out)
+    torch.cuda.synchronize()
+    sa, sb = torch.cuda.Stream(), torch.cuda.Stream()
+    outs = [torch.empty_like(wa.q), torch.empty_like(wb.q)]
+    for _ in range(3):
+        with torch.cuda.stream(sa):
+            ops.paged_attn_decode(wa.q, wa.k_cache, wa.v_cache, wa.block_table, wa.context_lens, wa.scale, outs[0],
+                                  ws_a, split_workgroups=37)
+        with torch.cuda.stream(sb):
+            ops.paged_attn_decode(wb.q, wb.k_cache, wb.v_cache, wb.block_table, wb.context_lens, wb.scale, outs[1],
+                                  ws_b, split_workgroups=256)
+    torch.cuda.synchronize()
+    for wl, got, ref in ((wa, outs[0], serial[0]), (wb, outs[1], serial[1])):
+        assert np.array_equal(bits(got), bits(ref))
+        assert float(np.abs(f32(got) - oracle_decode(wl)).max()) <= ATTN_ATOL
+
+
+def test_split_then_merge_need_not_agree_on_a_setting(gpu):
+    """The merge phase locates the partial results from the workspace alone: a split launched with any
+    split count is merged correctly by the same merge call."""
+    wl = workloads.make_decode_workload("sm", [2000, 300, 4096, 1], 32, 8, seed=13).to(gpu)
+    ws = ops.decode_workspace(gpu, 4, 32, 8, 128)
+    want = oracle_decode(wl)
+    for w in (1, 5, 64, 1024):
+        out = torch.full_like(wl.q, float("nan"))
+        ops.paged_attn_decode_split(wl.q, wl.k_cache, wl.v_cache, wl.block_table, wl.context_lens, wl.scale, ws,
+                                    split_workgroups=w)
+        ops.paged_attn_decode_merge(out, wl.context_lens, 8, ws)
+        torch.cuda.synchronize()
+        assert float(np.abs(f32(out) - want).max()) <= ATTN_ATOL
+
+
+def test_length_beyond_the_table_is_cut_to_the_table(gpu):
+    """A context length larger than table_cols * block_size (a corrupt length) must not make the kernel
+    read block ids past its table row: the row is attended as if it were table_cols blocks long."""
+    wl = workloads.make_decode_workload("clamp", [512, 700, 256], 16, 8, seed=14).to(gpu)
+    cols = wl.block_table.shape[1]                      # 3 blocks
+    full = [cols * 256] * 3
+    bad = torch.tensor([10 ** 6, 2 ** 31 - 1, cols * 256 + 1], dtype=torch.int32, device=gpu)
+    bt = wl.block_table.clamp(min=0).contiguous()       # every entry of the row is a real block
+    out_bad = torch.empty_like(wl.q)
+    out_full = torch.empty_like(wl.q)
+    ops.paged_attn_decode(wl.q, wl.k_cache, wl.v_cache, bt, bad, wl.scale, out_bad)
+    ops.paged_attn_decode(wl.q, wl.k_cache, wl.v_cache, bt, torch.tensor(full, dtype=torch.int32, device=gpu),
+                          wl.scale, out_full)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(out_bad), bits(out_full))
