@@ -161,6 +161,30 @@ int infer_paged_decode_merge_bf16(void* out, int64_t out_stride0,
                                   const void* workspace, size_t workspace_bytes,
                                   void* stream);
 
+/* infer_paged_decode_bf16 for callers that cannot allocate and have no workspace to bring: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in
+ * the reference.  Same arguments, result and kernels as infer_paged_decode_bf16 with
+ * split_workgroups = 0, but the split-KV partial results go to a fixed array in the library's device
+ * image (16 MiB per GPU the library runs on, held until the process ends) instead of a workspace.
+ * The call allocates nothing and frees nothing.  Shapes whose partial results do not fit return
+ * INFER_KV_EWORKSPACE: the need is about Hkv * (CUs * 8 / Hkv + batch) * 520 * G bytes, i.e. 5.3 MB at
+ * batch 64, Hq/Hkv = 32/8 and 8.8 MB at batch 8, 64/8 on 256 compute units, against the
+ * INFER_KV_DECODE_NOALLOC_SCRATCH_BYTES of the array.  The array keeps the last
+ * call's contents and needs no clearing (every record that is read was written by the same call).
+ * All calls on one GPU share it: calls that overlap on one GPU (two streams, two threads) race;
+ * calls ordered on one stream are safe.  The first call on a device resolves the array's address
+ * (hipGetSymbolAddress); make that call outside stream capture. */
+#define INFER_KV_DECODE_NOALLOC_SCRATCH_BYTES ((size_t)16 << 20)
+int infer_paged_decode_noalloc_bf16(const void* q, int64_t q_stride0,
+                                    const void* k_cache, const void* v_cache,
+                                    int64_t cache_block_stride, int64_t cache_token_stride,
+                                    void* out, int64_t out_stride0,
+                                    const int32_t* block_table, int64_t bt_stride0, int64_t table_cols,
+                                    const int32_t* context_lens,
+                                    int64_t batch, int64_t num_q_heads, int64_t num_kv_heads,
+                                    int64_t head_dim, int64_t block_size, int64_t num_blocks,
+                                    float scale, void* stream);
+
 /* ------------------------------------------------------------------ 2b. paged varlen prefill attention
  * Replaces flash_attn_varlen_func(Q, K, V, max_seqlen_q, cu_seqlens_q, max_seqlen_k, cu_seqlens_k,
  * softmax_scale, causal=True, block_table) at infer/ops/attention.py:110-116.

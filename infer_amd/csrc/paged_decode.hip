@@ -768,6 +768,36 @@ int launch_merge(void* out, int64_t out_stride0, const int32_t* context_lens, in
 
 }  // namespace
 
+// Scratch of infer_paged_decode_noalloc_bf16: the split-KV partial results of one call.  Every device
+// the library runs on holds its own copy of this array, at its own address, until the process ends.
+// In host code the array's NAME is only a handle for hipGetSymbolAddress, never a device address.
+constexpr size_t kNoAllocScratchBytes = INFER_KV_DECODE_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char infer_kv_decode_scratch[kNoAllocScratchBytes];
+
+namespace {
+
+// Device address of the scratch array on the current device, resolved once per device.
+int noalloc_scratch(void** out) {
+    static void* ptrs[kMaxDevices] = {nullptr};
+    static bool known[kMaxDevices] = {false};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return INFER_KV_EUNSUPPORTED;
+    if (!known[dev]) {      // a race between two first calls resolves the same address twice
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(infer_kv_decode_scratch));
+        if (e != hipSuccess) return (int)e;
+        if (p == nullptr) return INFER_KV_EINVAL;
+        ptrs[dev] = p;
+        __atomic_store_n(&known[dev], true, __ATOMIC_RELEASE);
+    }
+    *out = ptrs[dev];
+    return INFER_KV_OK;
+}
+
+}  // namespace
+
 extern "C" {
 
 size_t infer_paged_decode_workspace_bytes(int64_t max_batch, int64_t num_q_heads, int64_t num_kv_heads,
@@ -833,6 +863,32 @@ int infer_paged_decode_bf16(const void* q, int64_t q_stride0, const void* k_cach
     rc = launch_split(c, L, ws, workspace, (hipStream_t)stream);
     if (rc) return rc;
     return launch_merge(out, out_stride0, context_lens, batch, num_q_heads, num_kv_heads, ws, workspace,
+                        (hipStream_t)stream);
+}
+
+int infer_paged_decode_noalloc_bf16(const void* q, int64_t q_stride0, const void* k_cache, const void* v_cache,
+                                    int64_t cache_block_stride, int64_t cache_token_stride, void* out,
+                                    int64_t out_stride0, const int32_t* block_table, int64_t bt_stride0,
+                                    int64_t table_cols, const int32_t* context_lens, int64_t batch,
+                                    int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t block_size,
+                                    int64_t num_blocks, float scale, void* stream) {
+    const DecodeCall c{q, q_stride0, k_cache, v_cache, cache_block_stride, cache_token_stride, block_table, bt_stride0,
+                       table_cols, context_lens, batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks,
+                       scale};
+    void* scratch = nullptr;
+    int rc = noalloc_scratch(&scratch);
+    if (rc) return rc;
+    Launch L;
+    rc = check_split(c, /*split_workgroups=*/0, scratch, &L);
+    if (rc) return rc;
+    rc = check_out(out, out_stride0, num_q_heads);
+    if (rc) return rc;
+    // laid out for the split count this call launches, not for the largest one a workspace allows
+    const DecodeWorkspace ws = decode_workspace_layout(batch, num_q_heads / num_kv_heads, num_kv_heads, L.W);
+    if (ws.total_bytes > kNoAllocScratchBytes) return INFER_KV_EWORKSPACE;
+    rc = launch_split(c, L, ws, scratch, (hipStream_t)stream);
+    if (rc) return rc;
+    return launch_merge(out, out_stride0, context_lens, batch, num_q_heads, num_kv_heads, ws, scratch,
                         (hipStream_t)stream);
 }
 

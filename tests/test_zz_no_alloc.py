@@ -1,0 +1,55 @@
+"""The decode entry point that allocates nothing (infer_paged_decode_noalloc_bf16) against the
+workspace-taking entry point it shares its kernels with: same bits, on two calls in a row, the
+second with a smaller input, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from infer_amd import _lib, workloads
+from tests.helpers import ATTN_ATOL, bits, f32, oracle_decode
+
+pytestmark = pytest.mark.gpu
+
+
+def _call(entry, wl, out, workspace=None):
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    nblk, bs, hkv, d = wl.k_cache.shape
+    b, hq, _ = wl.q.shape
+    head = (wl.q.data_ptr(), wl.q.stride(0), wl.k_cache.data_ptr(), wl.v_cache.data_ptr(), wl.k_cache.stride(0),
+            wl.k_cache.stride(1), out.data_ptr(), out.stride(0), wl.block_table.data_ptr(), wl.block_table.stride(0),
+            wl.block_table.shape[1], wl.context_lens.data_ptr(), b, hq, hkv, d, bs, nblk, float(wl.scale))
+    if entry == "noalloc":
+        return lib.infer_paged_decode_noalloc_bf16(*head, stream)
+    return lib.infer_paged_decode_bf16(*head, 0, workspace.data_ptr(), workspace.numel(), stream)
+
+
+def test_two_calls_in_a_row_match_the_workspace_entry_point(gpu):
+    lib = _lib.load()
+    big = workloads.make_decode_workload("na-big", [1500, 37, 2300, 256, 700, 4096, 1023, 90] * 4, 32, 8, seed=21).to(gpu)
+    small = workloads.make_decode_workload("na-small", [300, 1, 64], 32, 8, seed=22).to(gpu)
+    ws = torch.empty(lib.infer_paged_decode_workspace_bytes(32, 32, 8, 128), dtype=torch.uint8, device=gpu)
+    for wl in (big, small):                       # second call: smaller input, scratch still holds the first call's records
+        want = torch.empty_like(wl.q)
+        got = torch.full_like(wl.q, float("nan"))
+        assert _call("workspace", wl, want, ws) == 0
+        assert _call("noalloc", wl, got) == 0
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(got), bits(want)), wl.name
+        assert float(np.abs(f32(got) - oracle_decode(wl)).max()) <= ATTN_ATOL
+
+
+def test_allocates_nothing_and_rejects_what_does_not_fit(gpu):
+    wl = workloads.make_decode_workload("na-mem", [700, 33], 64, 8, seed=23).to(gpu)
+    out = torch.empty_like(wl.q)
+    assert _call("noalloc", wl, out) == 0          # first call on the device resolves the scratch address
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info(gpu)[0]
+    for _ in range(5):
+        assert _call("noalloc", wl, out) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info(gpu)[0] == free_before
+    assert float(np.abs(f32(out) - oracle_decode(wl)).max()) <= ATTN_ATOL
+    # partial results of batch 4096 at 32/8 heads need 8 * (256 + 4096) records of 2080 bytes = 72 MB > 16 MiB
+    many = workloads.make_decode_workload("na-many", [5] * 4096, 32, 8, nblk=4100, bs=32, seed=24).to(gpu)
+    assert _call("noalloc", many, torch.empty_like(many.q)) == -3
