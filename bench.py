@@ -280,7 +280,8 @@ def main():
                          "probe library, same timing method) and print it as JSON; no KV-cache kernel runs")
     ap.add_argument("--counters", action="store_true",
                     help="short untimed run for `rocprofv3 --pmc`: a 1 GiB plain copy (x3), the decode op (x5), "
-                         "a prefill-sized append (x3), its read half and its write half (x3 each)")
+                         "a prefill-sized append (x3), its read half and its write half (x3 each), the fused "
+                         "norm + RoPE + append (x3) and the prefill attention (x3) of the same step")
     ap.add_argument("--append-sweep", action="store_true",
                     help="KV append rate against the number of rows (64 ... 65,536), printed as JSON")
     ap.add_argument("--decode-curve", action="store_true", help="only the decode curve, printed as JSON")
@@ -441,9 +442,28 @@ def main():
         for _ in range(3):
             _lib.check(probe.infer_kv_probe_append_write_half(p3.k_cache.data_ptr(), p3.v_cache.data_ptr(),
                                                               p3.slot_mapping.data_ptr(), n3, slots3, stream), "probe")
+        n_q = int(p3.q.shape[0])
+        qkv = torch.randn((n_q, (hq + 2 * hkv) * d), dtype=torch.bfloat16, device=dev)
+        q_, k_, v_ = (t.view(n_q, -1, d) for t in qkv.split([hq * d, hkv * d, hkv * d], dim=-1))
+        w_ = torch.ones(d, dtype=torch.bfloat16, device=dev)
+        cs_ = torch.randn((4096, d), dtype=torch.bfloat16, device=dev)
+        pos_ = torch.randint(0, 4096, (n_q,), device=dev)
+        sl_ = p3.slot_mapping[p3.row_of_query].contiguous()
+        for _ in range(3):
+            ops.qk_norm_rope_store_kvcache(q_, k_, v_, pos_, w_, w_, 1e-6, cs_, p3.k_cache, p3.v_cache, sl_,
+                                           write_key=False)
+        ops.store_kvcache(p3.k_new, p3.v_new, p3.k_cache, p3.v_cache, p3.slot_mapping)
+        for _ in range(3):
+            ops.flash_attn_varlen_func(p3.q, p3.k_cache, p3.v_cache, max_seqlen_q=p3.max_seqlen_q,
+                                       cu_seqlens_q=p3.cu_seqlens_q, max_seqlen_k=p3.max_seqlen_k,
+                                       cu_seqlens_k=p3.cu_seqlens_k, softmax_scale=p3.scale, causal=True,
+                                       block_table=p3.block_table)
         torch.cuda.synchronize()
+        pairs = sum((n - c) * c + (n - c) * (n - c + 1) // 2 for n, c in zip(p3.lengths, p3.cached))
         print(json.dumps({"counters_run": True, "copy_bytes": 1 << 30, "decode_algorithmic_bytes": wl.decode_bytes,
-                          "append_algorithmic_bytes": p3.append_bytes}))
+                          "append_algorithmic_bytes": p3.append_bytes,
+                          "fused_algorithmic_bytes": n_q * (2 * hq * d * 2 + 4 * hkv * d * 2),
+                          "prefill_flops": 4 * p3.num_q_heads * p3.head_dim * pairs}))
         return
 
     wl = workloads.cfg2().to(dev)                   # the headline workload: seeded on the CPU, then moved
