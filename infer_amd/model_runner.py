@@ -69,6 +69,12 @@ class ModelRunner:
         seqs = [Sequence([0] * max_len, SamplingParams(temperature=0.7, max_tokens=512)) for _ in range(num_seqs)]
         self.run(seqs, True)
         torch.cuda.empty_cache()
+        # what a decode step needs beyond the model is allocated now, before the pool is sized from what
+        # is left: the split-KV workspace for the largest batch and the split-K GEMM's partial sums
+        hf = self.config.hf_config
+        ops.decode_workspace(self.device, min(self.config.max_num_seqs, 512), hf.num_attention_heads,
+                             hf.num_key_value_heads, hf.head_dim)
+        ops._gemm_workspace(self.device, 64 << 20)
 
     def allocate_kv_cache(self):
         config, hf = self.config, self.config.hf_config

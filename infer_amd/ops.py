@@ -415,6 +415,25 @@ _linear_choice: dict = {}
 _linear_timings: dict = {}      # (device, batch bucket, N, K) -> (vendor ms, own ms), for inspection
 _flush_buffers: dict = {}
 
+# Weight matrices with at most this many rows go to the split-K kernel at decode batch sizes: the vendor
+# GEMM has too few output tiles to fill the chip there (o_proj, down_proj: 4096 rows = 32 tiles of 128 on
+# 256 compute units, 27 and 68 us against 22 and 38), and is ahead on every wider projection measured
+# (qkv 6144, gate_up 24576, lm_head 151936 rows) and on short reductions (K below 2048).  On the three
+# published Qwen3 shapes the rule picks what a cold-cache timing of both kernels picks, within 2.5 %
+# of a decode step on the smallest.
+SKINNY_MAX_ROWS = 5120
+
+
+def _linear_mode() -> str:
+    """``INFER_AMD_LINEAR``: ``static`` (default: the fixed rule above, the same kernel for a shape in every
+    process), ``vendor`` (never the split-K kernel), ``measure`` (time both once per shape with cold caches and
+    keep the faster: a tuning aid, not reproducible from run to run)."""
+    import os
+    mode = os.environ.get("INFER_AMD_LINEAR", "static")
+    if mode not in ("static", "vendor", "measure"):
+        raise RuntimeError(f"INFER_AMD_LINEAR must be static, vendor or measure, not {mode!r}")
+    return mode
+
 
 def _time_cold(fn, device, reps: int = 6) -> float:
     """Median GPU time of ``fn`` with the caches flushed before every launch (the weights of a decode
@@ -437,28 +456,33 @@ def _time_cold(fn, device, reps: int = 6) -> float:
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, defer: bool = False):
-    """``F.linear(x, weight)`` that sends decode-sized batches to whichever of the vendor GEMM and the
-    split-K weight-streaming kernel is faster for the shape.  The choice is measured once per
-    (device, batch bucket, N, K) with cold caches and kept for the life of the process, so every
-    later call for the shape runs the same kernel; while a HIP graph is being captured nothing is
-    measured (an unknown shape takes the vendor GEMM)."""
+    """``F.linear(x, weight)`` that sends decode-sized batches over narrow weight matrices to the split-K
+    weight-streaming kernel and everything else to the vendor GEMM.  The choice is a fixed rule on the
+    shape (see ``_linear_mode`` for the alternatives), so a shape runs the same kernel, with the same
+    rounding, in every process and inside and outside a captured graph."""
     if x.dim() != 2 or not x.is_cuda or x.dtype != torch.bfloat16:
         return torch.nn.functional.linear(x, weight)
     m, k = x.shape
     n = weight.shape[0]
     if not skinny_linear_supported(m, n, k) or not weight.is_contiguous() or x.stride(1) != 1:
         return torch.nn.functional.linear(x, weight)
-    bucket = 16 if m <= 16 else 32 if m <= 32 else 64 if m <= 64 else 128
-    key = (str(x.device), bucket, n, k)
-    use = _linear_choice.get(key)
-    if use is None:
-        if torch.cuda.is_current_stream_capturing():
-            return torch.nn.functional.linear(x, weight)
-        probe = x if m == bucket else torch.zeros((bucket, k), dtype=x.dtype, device=x.device)
-        t_lib = _time_cold(lambda: torch.nn.functional.linear(probe, weight), x.device)
-        t_own = _time_cold(lambda: skinny_linear(probe, weight), x.device)
-        _linear_timings[key] = (t_lib, t_own)
-        use = _linear_choice[key] = bool(t_own < 0.95 * t_lib)
+    mode = _linear_mode()
+    if mode == "vendor":
+        return torch.nn.functional.linear(x, weight)
+    if mode == "static":
+        use = n <= SKINNY_MAX_ROWS and k >= 2048
+    else:
+        bucket = 16 if m <= 16 else 32 if m <= 32 else 64 if m <= 64 else 128
+        key = (str(x.device), bucket, n, k)
+        use = _linear_choice.get(key)
+        if use is None:
+            if torch.cuda.is_current_stream_capturing():
+                return torch.nn.functional.linear(x, weight)
+            probe = x if m == bucket else torch.zeros((bucket, k), dtype=x.dtype, device=x.device)
+            t_lib = _time_cold(lambda: torch.nn.functional.linear(probe, weight), x.device)
+            t_own = _time_cold(lambda: skinny_linear(probe, weight), x.device)
+            _linear_timings[key] = (t_lib, t_own)
+            use = _linear_choice[key] = bool(t_own < 0.95 * t_lib)
     if not use:
         return torch.nn.functional.linear(x, weight)
     # ``defer``: the caller hands the result straight to ``rms_norm``, which adds the partial sums itself
