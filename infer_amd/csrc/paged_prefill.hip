@@ -116,10 +116,20 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane >> 4, n = lane & 15;
-    const int b = blockIdx.y;
+    // Workgroups are dealt to the eight dies (XCDs) round-robin by their linear id, and each die has an L2
+    // of its own.  The linear id is therefore remapped so that die k works through the k-th contiguous
+    // eighth of the (query block, sequence, KV head) space: the workgroups that read the same keys sit
+    // behind one L2 and the K/V tiles of a (sequence, KV head) are fetched from HBM once, not once per die.
+    const unsigned wg_total = gridDim.x * gridDim.y * gridDim.z;
+    const unsigned wg_linear = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+    const unsigned die = wg_linear & 7u, per_die = wg_total >> 3, extra = wg_total & 7u;
+    const unsigned wg_id = __builtin_amdgcn_readfirstlane(die * per_die + (die < extra ? die : extra) + (wg_linear >> 3));
+    const int block_x = (int)(wg_id % gridDim.x);
+    const int b = (int)((wg_id / gridDim.x) % gridDim.y);
+    const int block_z = (int)(wg_id / (gridDim.x * gridDim.y));
     const int parts = a.group / kHeads;                    // workgroups that share one KV head
-    const int kvh = blockIdx.z / parts;
-    const int head = kvh * a.group + (blockIdx.z % parts) * kHeads + (QB == 1 ? wave : wave % kHeads);
+    const int kvh = block_z / parts;
+    const int head = kvh * a.group + (block_z % parts) * kHeads + (QB == 1 ? wave : wave % kHeads);
     const int qb = QB == 1 ? 0 : wave / kHeads;            // query block of this wavefront inside the workgroup
 
     const int q_beg = a.cu_q[b], q_end = a.cu_q[b + 1];
@@ -128,7 +138,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     int sk = k_end - k_beg;
     if (a.bt != nullptr && sk > a.max_sk) sk = a.max_sk;   // a corrupt length cannot run the gather past its table row
     // late query blocks see the most keys: hand them out first so the long workgroups start early
-    const int wg_q0 = (int)(gridDim.x - 1 - blockIdx.x) * QB * kQBlock;
+    const int wg_q0 = (int)(gridDim.x - 1 - block_x) * QB * kQBlock;
     if (wg_q0 >= sq) return;
     const int q0 = wg_q0 + qb * kQBlock;
     const bool live = QB == 1 || q0 < sq;   // a trailing wavefront may have no queries: it only helps to fetch
