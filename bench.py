@@ -520,25 +520,31 @@ def main():
 
     ap_ms = gpu_time_ms(append_step, max(args.steps, 48), reps)
     append_gbs = p3.append_bytes / (ap_ms * 1e-3) / 1e9
-    # the two halves of that append on their own (probe library): what its reads and its writes cost alone
-    probe = load_probe_library()
-    stream = torch.cuda.current_stream().cuda_stream
-    sink = torch.zeros(4, dtype=torch.uint8, device=dev)
-    n3, slots3 = int(p3.slot_mapping.numel()), p3.k_cache.shape[0] * 256
+    # the two halves of that append on their own (probe library): what its reads and its writes cost alone.
+    # The probe library is measurement scaffolding: without it the two figures are left out, nothing else.
+    rd_ms = wr_ms = None
+    try:
+        probe = load_probe_library()
+    except (ImportError, OSError, AttributeError):
+        probe = None
+    if probe is not None:
+        stream = torch.cuda.current_stream().cuda_stream
+        sink = torch.zeros(4, dtype=torch.uint8, device=dev)
+        n3, slots3 = int(p3.slot_mapping.numel()), p3.k_cache.shape[0] * 256
 
-    def read_half():
-        j = jt[0] % reps
-        jt[0] += 1
-        probe.infer_kv_probe_append_read_half(srcs[j][0].data_ptr(), srcs[j][1].data_ptr(), p3.slot_mapping.data_ptr(),
-                                              n3, slots3, sink.data_ptr(), stream)
+        def read_half():
+            j = jt[0] % reps
+            jt[0] += 1
+            probe.infer_kv_probe_append_read_half(srcs[j][0].data_ptr(), srcs[j][1].data_ptr(),
+                                                  p3.slot_mapping.data_ptr(), n3, slots3, sink.data_ptr(), stream)
 
-    def write_half():
-        j = jt[0] % reps
-        jt[0] += 1
-        probe.infer_kv_probe_append_write_half(dsts[j][0].data_ptr(), dsts[j][1].data_ptr(), p3.slot_mapping.data_ptr(),
-                                               n3, slots3, stream)
-    rd_ms = gpu_time_ms(read_half, 48, reps)
-    wr_ms = gpu_time_ms(write_half, 48, reps)
+        def write_half():
+            j = jt[0] % reps
+            jt[0] += 1
+            probe.infer_kv_probe_append_write_half(dsts[j][0].data_ptr(), dsts[j][1].data_ptr(),
+                                                   p3.slot_mapping.data_ptr(), n3, slots3, stream)
+        rd_ms = gpu_time_ms(read_half, 48, reps)
+        wr_ms = gpu_time_ms(write_half, 48, reps)
 
     # fused QK-norm + RoPE + append (one launch for the four steps in front of attention), over rotated
     # qkv buffers and cache pairs (> 512 MB in total) so that every launch reads and writes HBM
@@ -593,7 +599,8 @@ def main():
                    "prefill_rows": int(p3.slot_mapping.numel()), "prefill_bytes": p3.append_bytes,
                    "prefill_us": round(ap_ms * 1e3, 2), "prefill_GBps": round(append_gbs, 1),
                    "prefill_frac_of_peak": round(append_gbs / HBM_PEAK_GBS, 4),
-                   "read_half_alone_us": round(rd_ms * 1e3, 2), "write_half_alone_us": round(wr_ms * 1e3, 2)},
+                   "read_half_alone_us": round(rd_ms * 1e3, 2) if rd_ms else None,
+                   "write_half_alone_us": round(wr_ms * 1e3, 2) if wr_ms else None},
     }
     line["prefill_attention"] = {"workload": "cfg3: 16 prompts U[64,2048], 0-50 % cached, causal over the paged cache",
                                  "query_tokens": int(p3.q.shape[0]), "ms": round(pf_ms, 4),

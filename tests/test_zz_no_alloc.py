@@ -53,3 +53,40 @@ def test_allocates_nothing_and_rejects_what_does_not_fit(gpu):
     # partial results of batch 4096 at 32/8 heads need 8 * (256 + 4096) records of 2080 bytes = 72 MB > 16 MiB
     many = workloads.make_decode_workload("na-many", [5] * 4096, 32, 8, nblk=4100, bs=32, seed=24).to(gpu)
     assert _call("noalloc", many, torch.empty_like(many.q)) == -3
+
+
+def test_replays_inside_a_hip_graph(gpu):
+    """What the entry point is for: a captured decode step that may not allocate.  The graph is replayed
+    with new lengths, tables and queries in its static buffers, with eager work in between; every replay
+    must give the bits of the eager workspace call on the same inputs."""
+    lib = _lib.load()
+    shapes = ([900, 33, 2047, 256], [64, 1300, 5, 700], [1, 1, 4096, 12])
+    wls = [workloads.make_decode_workload(f"na-g{i}", lens, 32, 8, nblk=40, seed=30 + i).to(gpu)
+           for i, lens in enumerate(shapes)]
+    st = wls[0]
+    static = workloads.DecodeWorkload(**{k: (v.clone() if isinstance(v, torch.Tensor) else v)
+                                         for k, v in st.__dict__.items()})
+    cols = max(w.block_table.shape[1] for w in wls)
+    static.block_table = torch.zeros((4, cols), dtype=torch.int32, device=gpu)
+    out = torch.empty_like(static.q)
+    assert _call("noalloc", wls[0], torch.empty_like(st.q)) == 0      # resolves the scratch address outside capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            assert _call("noalloc", static, out) == 0
+    torch.cuda.synchronize()
+    ws = torch.empty(lib.infer_paged_decode_workspace_bytes(4, 32, 8, 128), dtype=torch.uint8, device=gpu)
+    for wl in wls + wls[::-1]:
+        static.q.copy_(wl.q)
+        static.k_cache.copy_(wl.k_cache)
+        static.v_cache.copy_(wl.v_cache)
+        static.context_lens.copy_(wl.context_lens)
+        static.block_table.zero_()
+        static.block_table[:, :wl.block_table.shape[1]] = wl.block_table.clamp(min=0)
+        graph.replay()
+        want = torch.empty_like(wl.q)
+        assert _call("workspace", wl, want, ws) == 0                     # eager work between the replays
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(out), bits(want)), wl.name
