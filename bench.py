@@ -65,6 +65,7 @@ def load_probe_library():
         "infer_kv_probe_read_streaming": [vp, sz, vp, ctypes.c_int, vp],
         "infer_kv_probe_copy": [vp, vp, sz, ctypes.c_int, vp],
         "infer_kv_probe_copy_rows": [vp, vp, sz, vp],
+        "infer_kv_probe_read_kv_pattern": [vp, vp, sz, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, ctypes.c_int, vp],
         "infer_kv_probe_append_read_half": [vp, vp, vp, i64, i64, vp, vp],
         "infer_kv_probe_append_write_half": [vp, vp, vp, i64, i64, vp],
     }.items():
@@ -359,6 +360,15 @@ def main():
                 ms = gpu_time_ms(cp(wg), 30, 3)
                 res[f"copy_{label}_{wg}wg_GBps_read_plus_write"] = round(2 * nbytes / ms / 1e6, 1)
             del bufs, dst, dsts
+        # the decode kernel's two read streams (K and V, 1 GiB each) by access pattern and streaming hint
+        tokens = 1 << 19
+        kbuf = torch.empty(tokens * 2048, dtype=torch.uint8, device=dev).random_(0, 255)
+        vbuf = torch.empty(tokens * 2048, dtype=torch.uint8, device=dev).random_(0, 255)
+        for whole, kh, vh in ((0, 0, 0), (0, 0, 1), (0, 1, 1), (1, 0, 0), (1, 0, 1), (1, 1, 0), (1, 1, 1)):
+            ms = gpu_time_ms(lambda: _lib.check(lib.infer_kv_probe_read_kv_pattern(
+                kbuf.data_ptr(), vbuf.data_ptr(), tokens, whole, kh, vh, sink.data_ptr(), 256, stream), "probe"), 8, 2)
+            res[f"kv_streams_2GiB_K_{'rows' if whole else 'mfma_pattern'}_{'hint' if kh else 'plain'}_V_rows_"
+                f"{'hint' if vh else 'plain'}_GBps"] = round(2 * tokens * 2048 / ms / 1e6, 1)
         print(json.dumps(res))
         return
     if args.append_sweep:

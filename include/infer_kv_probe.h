@@ -27,6 +27,14 @@ int infer_kv_probe_copy(const void* src, void* dst, size_t bytes, int workgroups
 /* a copy with one wavefront per 4 KiB and no loop (whole 4 KiB pieces only) */
 int infer_kv_probe_copy_rows(const void* src, void* dst, size_t bytes, void* stream);
 
+/* The two read streams of the decode kernel without its arithmetic: `tokens` rows of 2 KiB (8 KV heads of
+ * 256 B) in each of k and v, one wavefront per KV head, 32-token steps in contiguous per-workgroup shares.
+ * V is read as whole rows; K in the decode kernel's MFMA-operand pattern (16 tokens x 64 B per
+ * instruction) or, with k_whole_rows, as whole rows too.  k_hint / v_hint put the streaming
+ * (nontemporal) hint on the loads of that stream. */
+int infer_kv_probe_read_kv_pattern(const void* k, const void* v, size_t tokens, int k_whole_rows, int k_hint,
+                                   int v_hint, void* sink4, int workgroups, void* stream);
+
 /* The two halves of infer_kv_append_bf16 for rows of 2 KiB (dkv = 1024), contiguous sources: the
  * first loads the K and V row of every row with a valid slot and stores nothing, the second stores
  * a K and a V row to the slot of every such row and loads nothing. */

@@ -67,6 +67,50 @@ __global__ void __launch_bounds__(256) stream_copy_rows_kernel(const u32x4* __re
     for (int u = 0; u < 4; ++u) __builtin_nontemporal_store(r[u], dst + base + lane + 64 * u);
 }
 
+// The decode kernel's two read streams without its arithmetic: eight wavefronts per workgroup, one per KV
+// head, steps of 32 tokens over rows of 2 KiB (8 heads x 256 B), two steps requested before either is
+// consumed.  V rows are always read as whole rows (four tokens x 256 B per instruction).  K is read either
+// in the MFMA-operand pattern of the decode kernel (KPAT 0: 16 tokens x 64 B per instruction, so each
+// 128-byte line is touched by two instructions) or as whole rows like V (KPAT 1); KNT / VNT put the
+// streaming hint on the K / V loads.
+template <int KPAT, bool KNT, bool VNT>
+__global__ void __launch_bounds__(512) kv_pattern_read_kernel(const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
+                                                               size_t tokens, uint32_t* sink) {
+    const int lane = threadIdx.x & 63, h = threadIdx.x >> 6;
+    const int g = lane >> 4, n = lane & 15;
+    const size_t per = tokens / gridDim.x / 32;      // steps per workgroup
+    const size_t s0 = per * blockIdx.x;
+    const uint32_t tok = 1024;                       // elements per token row
+    const uint32_t k_lane = (8 * (n >> 2) + (n & 3)) * tok + 8 * g;
+    const uint32_t v_lane = g * tok + 8 * n;
+    uint32_t acc = 0;
+    for (size_t s = s0; s + 2 <= s0 + per; s += 2) {
+        u32x4 r[2][16];
+#pragma unroll
+        for (int dd = 0; dd < 2; ++dd) {
+            const uint16_t* kb = k + (s + dd) * 32 * tok + h * 128;
+            const uint16_t* vb = v + (s + dd) * 32 * tok + h * 128;
+            if (KPAT == 0) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        r[dd][t * 4 + j] = probe_load<KNT>(reinterpret_cast<const u32x4*>(kb + t * 4 * tok + k_lane + 32 * j));
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) r[dd][i] = probe_load<KNT>(reinterpret_cast<const u32x4*>(kb + i * 4 * tok + v_lane));
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) r[dd][8 + i] = probe_load<VNT>(reinterpret_cast<const u32x4*>(vb + i * 4 * tok + v_lane));
+        }
+#pragma unroll
+        for (int dd = 0; dd < 2; ++dd)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc ^= fold(r[dd][i]);
+    }
+    if (acc == 0x9e3779b9u) *sink = acc;   // keeps the loads alive; practically never true
+}
+
 // Read half of the KV append: every row with a valid slot is loaded (K and V, 2 KiB each), nothing
 // is stored.  One wavefront per row, as the append kernel for few rows.
 __global__ void __launch_bounds__(256) append_read_half_kernel(const u32x4* __restrict__ key, const u32x4* __restrict__ value,
@@ -105,6 +149,31 @@ __global__ void __launch_bounds__(256) append_write_half_kernel(u32x4* __restric
 }  // namespace
 
 extern "C" {
+
+int infer_kv_probe_read_kv_pattern(const void* k, const void* v, size_t tokens, int k_whole_rows, int k_hint, int v_hint,
+                                   void* sink4, int workgroups, void* stream) {
+    if (!k || !v || !sink4 || workgroups <= 0 || tokens < (size_t)workgroups * 64 || (((uintptr_t)k | (uintptr_t)v) & 15))
+        return INFER_KV_EINVAL;
+    const dim3 grid(workgroups), block(512);
+    hipStream_t st = (hipStream_t)stream;
+    const uint16_t* kp = (const uint16_t*)k;
+    const uint16_t* vp = (const uint16_t*)v;
+    uint32_t* sk = (uint32_t*)sink4;
+#define INFER_KV_PROBE_PATTERN(P, KN, VN) hipLaunchKernelGGL((kv_pattern_read_kernel<P, KN, VN>), grid, block, 0, st, kp, vp, tokens, sk)
+    const int sel = (k_whole_rows ? 4 : 0) | (k_hint ? 2 : 0) | (v_hint ? 1 : 0);
+    switch (sel) {
+        case 0: INFER_KV_PROBE_PATTERN(0, false, false); break;
+        case 1: INFER_KV_PROBE_PATTERN(0, false, true); break;
+        case 2: INFER_KV_PROBE_PATTERN(0, true, false); break;
+        case 3: INFER_KV_PROBE_PATTERN(0, true, true); break;
+        case 4: INFER_KV_PROBE_PATTERN(1, false, false); break;
+        case 5: INFER_KV_PROBE_PATTERN(1, false, true); break;
+        case 6: INFER_KV_PROBE_PATTERN(1, true, false); break;
+        default: INFER_KV_PROBE_PATTERN(1, true, true); break;
+    }
+#undef INFER_KV_PROBE_PATTERN
+    return (int)hipGetLastError();
+}
 
 int infer_kv_probe_append_read_half(const void* key, const void* value, const int32_t* slot_mapping, int64_t n_rows,
                                     int64_t num_slots, void* sink4, void* stream) {

@@ -25,7 +25,7 @@ def test_probe_library_exports_what_its_header_declares():
     """The measurement kernels live in a library of their own that only bench.py loads."""
     probe = ctypes.CDLL(os.path.join(ROOT, "infer_amd", "libinfer_kv_probe.so"))
     names = declared_functions("infer_kv_probe.h")
-    assert len(names) == 6
+    assert len(names) == 7
     for name in names:
         assert hasattr(probe, name), f"{name} declared in infer_kv_probe.h but not exported"
         assert not hasattr(_lib.load(), name), f"{name} must not be part of the product library"
