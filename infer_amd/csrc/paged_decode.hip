@@ -784,7 +784,7 @@ int noalloc_scratch(void** out) {
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return (int)e;
     if (dev < 0 || dev >= kMaxDevices) return INFER_KV_EUNSUPPORTED;
-    if (!known[dev]) {      // a race between two first calls resolves the same address twice
+    if (!__atomic_load_n(&known[dev], __ATOMIC_ACQUIRE)) {      // a race between two first calls resolves the same address twice
         void* p = nullptr;
         e = hipGetSymbolAddress(&p, HIP_SYMBOL(infer_kv_decode_scratch));
         if (e != hipSuccess) return (int)e;
