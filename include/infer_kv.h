@@ -65,6 +65,17 @@ int infer_kv_append_bf16(const void* key, int64_t key_stride0,
                          int64_t n_rows, int64_t dkv, int64_t num_slots,
                          void* stream);
 
+/* The dense per-sequence view that the getters of the reference's cache pool promise (Tensor<T>
+ * get_key_cache / get_value_cache, include/kvcache.hpp:47-48: [len, heads, head_size] contiguous): tokens
+ * 0 .. num_tokens-1 of ONE sequence gathered from the paged cache [num_blocks, block_size, dkv] through its
+ * block-table row (device memory, ceil(num_tokens / block_size) entries, clamped into [0, num_blocks)) into
+ * out [num_tokens, dkv].  The attention kernels never need it (they gather on the fly); it serves callers
+ * that want a sequence's K or V as one tensor, and is the inverse of the append (bit-exact copy).
+ * Requires dkv % 8 == 0 and 16-byte aligned pointers. */
+int infer_kv_gather_bf16(const void* cache, const int32_t* block_table_row,
+                         int64_t num_tokens, int64_t dkv, int64_t block_size, int64_t num_blocks,
+                         void* out, void* stream);
+
 /* ------------------------------------------------------------------ 1b. fused QK-norm + RoPE + KV append
  * Replaces, in one launch, the four steps in front of attention in QwenAttention.forward
  * (infer/models/Qwen3.py:113-131): q_norm and k_norm (RMSNorm.rms_forward, infer/ops/norm.py:63-73,

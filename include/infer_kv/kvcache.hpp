@@ -38,6 +38,8 @@ struct KVCachePoolConfig {
 };
 
 // What get_key_cache / get_value_cache hand out: the layer's cache and the sequence's blocks in it.
+// The paged kernels take it as it is; a caller that wants the reference's dense [len, heads, head_size]
+// tensor gets it with one infer_kv_gather_bf16 call on the view (block table copied to the device).
 template <typename T>
 struct PagedCacheView {
     T* base;                      // [num_blocks, block_size, num_heads, head_size] of this layer

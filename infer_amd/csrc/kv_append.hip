@@ -121,9 +121,39 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) kv_append_ring_kernel(App
     }
 }
 
+// The inverse direction for one sequence: token t of the sequence lives at block table[t / block_size],
+// offset t % block_size; one wavefront copies one token row into the dense output.
+__global__ void __launch_bounds__(64 * kWavesPerBlock) kv_gather_kernel(const u32x4* __restrict__ cache, const int32_t* __restrict__ table,
+                                                                        int64_t n_tokens, int row_chunks, int block_size,
+                                                                        int num_blocks, u32x4* __restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const int64_t t = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    if (t >= n_tokens) return;
+    int blk = __builtin_amdgcn_readfirstlane(table[t / block_size]);
+    blk = blk < 0 ? 0 : (blk >= num_blocks ? num_blocks - 1 : blk);     // a corrupt table cannot fault the GPU
+    const u32x4* src = cache + ((int64_t)blk * block_size + t % block_size) * row_chunks;
+    u32x4* dst = out + t * row_chunks;
+    for (int c = lane; c < row_chunks; c += 64) dst[c] = src[c];
+}
+
 }  // namespace
 
 extern "C" {
+
+int infer_kv_gather_bf16(const void* cache, const int32_t* block_table_row, int64_t num_tokens, int64_t dkv,
+                         int64_t block_size, int64_t num_blocks, void* out, void* stream) {
+    if (num_tokens == 0) return INFER_KV_OK;
+    if (!cache || !block_table_row || !out) return INFER_KV_EINVAL;
+    if (num_tokens < 0 || dkv <= 0 || block_size <= 0 || num_blocks <= 0) return INFER_KV_EINVAL;
+    if (block_size > 0x7fffffffLL || num_blocks > 0x7fffffffLL || dkv / 8 > 0x7fffffffLL) return INFER_KV_EINVAL;
+    if (dkv % 8 != 0 || (((uintptr_t)cache | (uintptr_t)out) & 15)) return INFER_KV_EALIGN;
+    const int64_t groups = (num_tokens + kWavesPerBlock - 1) / kWavesPerBlock;
+    if (groups > 0x7fffffffLL) return INFER_KV_EINVAL;
+    hipLaunchKernelGGL(kv_gather_kernel, dim3((unsigned)groups, 1, 1), dim3(64 * kWavesPerBlock, 1, 1), 0, (hipStream_t)stream,
+                       (const u32x4*)cache, block_table_row, num_tokens, (int)(dkv / 8), (int)block_size, (int)num_blocks,
+                       (u32x4*)out);
+    return (int)hipGetLastError();
+}
 
 int infer_kv_append_bf16(const void* key, int64_t key_stride0, const void* value, int64_t value_stride0,
                          void* k_cache, void* v_cache, const int32_t* slot_mapping, int64_t n_rows, int64_t dkv,

@@ -58,6 +58,22 @@ def store_kvcache(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor,
     _lib.check(rc, "store_kvcache")
 
 
+def gather_kvcache(cache: torch.Tensor, block_table_row: torch.Tensor, length: int) -> torch.Tensor:
+    """The first ``length`` tokens of one sequence as a dense ``[length, Hkv, D]`` tensor, gathered from the
+    paged ``cache`` ``[nblk, bs, Hkv, D]`` through the sequence's block-table row (int32, on the device): the
+    per-sequence tensor the getters of the reference's cache pool hand out (``include/kvcache.hpp:47-48``)."""
+    assert cache.dim() == 4 and cache.dtype == torch.bfloat16 and cache.is_contiguous()
+    nblk, bs, hkv, d = cache.shape
+    assert block_table_row.dtype == torch.int32 and block_table_row.dim() == 1 and block_table_row.is_contiguous()
+    assert 0 <= length <= block_table_row.numel() * bs
+    _require_gpu(cache, block_table_row)
+    out = torch.empty((length, hkv, d), dtype=cache.dtype, device=cache.device)
+    rc = _lib.load().infer_kv_gather_bf16(cache.data_ptr(), block_table_row.data_ptr(), length, hkv * d, bs, nblk,
+                                          out.data_ptr(), _stream_ptr(cache))
+    _lib.check(rc, "gather_kvcache")
+    return out
+
+
 def qk_norm_rope_store_kvcache(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, positions: torch.Tensor,
                                q_norm_weight: torch.Tensor, k_norm_weight: torch.Tensor, eps: float,
                                cos_sin_cache: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,

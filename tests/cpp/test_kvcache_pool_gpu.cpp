@@ -154,6 +154,24 @@ int main(int argc, char** argv) {
     HIP(hipMemcpy(other.data(), storage, other.size() * 2, hipMemcpyDeviceToHost));
     for (uint16_t x : other) CHECK(x == 0xffff);
 
+    // the dense [len, heads, head_size] tensor the reference's getters promise is one gather call on a view
+    std::vector<uint16_t> dense_k;
+    for (size_t i = 0; i < B; ++i) {
+        int32_t* d_row;
+        uint16_t* d_dense;
+        HIP(hipMalloc((void**)&d_row, kviews[i].num_blocks_used * 4));
+        HIP(hipMalloc((void**)&d_dense, (size_t)lens[i] * dkv * 2));
+        HIP(hipMemcpy(d_row, kviews[i].block_table, kviews[i].num_blocks_used * 4, hipMemcpyHostToDevice));
+        CHECK(infer_kv_gather_bf16(kviews[i].base, d_row, (int64_t)kviews[i].length, (int64_t)dkv, (int64_t)bs, (int64_t)nblk,
+                                   d_dense, nullptr) == 0);
+        std::vector<uint16_t> host((size_t)lens[i] * dkv);
+        HIP(hipMemcpy(host.data(), d_dense, host.size() * 2, hipMemcpyDeviceToHost));
+        dense_k.insert(dense_k.end(), host.begin(), host.end());
+        HIP(hipFree(d_row));
+        HIP(hipFree(d_dense));
+    }
+    CHECK(dense_k == k_rows);      // sequence-major rows, exactly what was appended
+
     std::vector<int64_t> meta = {(int64_t)B, (int64_t)Hq, (int64_t)Hkv, (int64_t)D, (int64_t)bs, (int64_t)nblk,
                                  (int64_t)cols, (int64_t)total};
     CHECK(!dump(outdir, "meta.i64", meta) && !dump(outdir, "q.u16", q) && !dump(outdir, "out.u16", out));

@@ -135,3 +135,29 @@ def test_scatter_then_gather_roundtrip_full_size(gpu):
     untouched[rows] = False
     assert torch.equal(kc.view(-1, width)[untouched], wl.k_cache.view(-1, width)[untouched])
     assert torch.equal(vc.view(-1, width)[untouched], wl.v_cache.view(-1, width)[untouched])
+
+
+def test_gather_is_the_inverse_of_the_append(gpu):
+    """ops.gather_kvcache hands out a sequence as the dense [len, Hkv, D] tensor the reference's pool getters
+    promise: bit-exact against the oracle's gather on every sequence of the prefill configuration after its
+    append, and equal to the rows that were appended."""
+    wl = workloads.cfg3().to(gpu)
+    kc, vc = wl.k_cache.clone(), wl.v_cache.clone()
+    ops.store_kvcache(wl.k_new, wl.v_new, kc, vc, wl.slot_mapping)
+    torch.cuda.synchronize()
+    hk, table = bits(kc), wl.block_table.cpu().numpy()
+    new_rows = wl.k_new[wl.row_of_query]                      # the appended rows in sequence order
+    at = 0
+    for i, (n, c) in enumerate(zip(wl.lengths, wl.cached)):
+        dense = ops.gather_kvcache(kc, wl.block_table[i].contiguous(), n)
+        torch.cuda.synchronize()
+        assert dense.shape == (n, wl.num_kv_heads, wl.head_dim)
+        assert np.array_equal(bits(dense), paged_ref.gather_sequence(hk, table[i], n))
+        assert torch.equal(dense[c:], new_rows[at:at + n - c])
+        at += n - c
+    assert ops.gather_kvcache(vc, wl.block_table[0].contiguous(), 0).shape[0] == 0
+    # a corrupt table entry is clamped into the pool instead of read out of bounds
+    bad = torch.tensor([10 ** 6, -5], dtype=torch.int32, device=gpu)
+    got = ops.gather_kvcache(kc, bad, 300)
+    torch.cuda.synchronize()
+    assert torch.equal(got[:256], kc[kc.shape[0] - 1]) and torch.equal(got[256:], kc[0, :44])

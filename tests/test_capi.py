@@ -67,6 +67,9 @@ def test_argument_errors_are_reported_before_anything_is_launched():
     p16 = (p + 15) & ~15
     assert lib.infer_kv_append_bf16(p16, 1024, p16, 1024, p16, p16, p16, 4, 1020, 256, None) == -2   # dkv % 8
     assert lib.infer_kv_append_bf16(p16 + 2, 1024, p16, 1024, p16, p16, p16, 4, 1024, 256, None) == -2
+    assert lib.infer_kv_gather_bf16(None, None, 5, 1024, 256, 4, None, None) == -1
+    assert lib.infer_kv_gather_bf16(None, None, 0, 1024, 256, 4, None, None) == 0
+    assert lib.infer_kv_gather_bf16(p16, p16, 5, 1020, 256, 4, p16, None) == -2
     assert lib.infer_paged_decode_bf16(None, 0, None, None, 0, 0, None, 0, None, 0, 1, None,
                                        1, 32, 8, 128, 256, 4, 1.0, 0, None, 0, None) == -1
     # the combined decode call rejects what its second launch would reject before the first is enqueued
