@@ -334,3 +334,29 @@ def test_length_beyond_the_table_is_cut_to_the_table(gpu):
                           wl.scale, out_full)
     torch.cuda.synchronize()
     assert np.array_equal(bits(out_bad), bits(out_full))
+
+
+@pytest.mark.parametrize("scale", [0.02, 0.3])
+def test_softmax_scale_is_honoured(gpu, scale):
+    """A scale other than head_dim ** -0.5 (the reference passes its own, infer/models/Qwen3.py:76)."""
+    wl = workloads.make_decode_workload("scale", [37, 300, 1025, 700], 32, 8, nblk=16, seed=31).to(gpu)
+    wl.scale = scale
+    check(wl)
+
+
+def test_query_and_output_rows_as_strided_views(gpu):
+    """Q as a column slice of the fused qkv matrix (infer/models/Qwen3.py:110-111) and the output as a
+    slice of a wider buffer: same bits as with contiguous tensors."""
+    wl = workloads.make_decode_workload("views", [37, 300, 1025, 700], 32, 8, nblk=16, seed=32).to(gpu)
+    want = gpu_decode(wl, splits=0)
+    b, hq, d = wl.q.shape
+    qkv = torch.randn((b, (hq + 16) * d), device=gpu).to(torch.bfloat16)
+    qkv[:, :hq * d] = wl.q.reshape(b, -1)
+    q_view = qkv.split([hq * d, 8 * d, 8 * d], dim=-1)[0].view(b, hq, d)
+    wide = torch.full((b, hq * d + 256), 7.0, dtype=torch.bfloat16, device=gpu)
+    out_view = wide[:, :hq * d].view(b, hq, d)
+    assert not q_view.is_contiguous() and not out_view.is_contiguous()
+    ops.paged_attn_decode(q_view, wl.k_cache, wl.v_cache, wl.block_table, wl.context_lens, wl.scale, out_view)
+    torch.cuda.synchronize()
+    assert torch.equal(out_view, want)
+    assert (wide[:, hq * d:] == 7.0).all()      # nothing written beside the output rows

@@ -165,3 +165,81 @@ def test_attention_module_prefill_then_decode(gpu):
                                        wl.block_table.cpu().numpy(), ctx.cpu().numpy(), wl.scale)
     assert np.abs(f32(o1).reshape(want1.shape) - want1).max() <= ATTN_ATOL
     reset_context()
+
+
+def _packed_case(gpu, lens_q, lens_k, hq, hkv, seed):
+    g = torch.Generator().manual_seed(seed)
+    d = 128
+    q = torch.randn((sum(lens_q), hq, d), generator=g).to(torch.bfloat16).to(gpu)
+    k = torch.randn((sum(lens_k), hkv, d), generator=g).to(torch.bfloat16).to(gpu)
+    v = torch.randn((sum(lens_k), hkv, d), generator=g).to(torch.bfloat16).to(gpu)
+    cu_q = torch.tensor(np.cumsum([0] + lens_q), dtype=torch.int32, device=gpu)
+    cu_k = torch.tensor(np.cumsum([0] + lens_k), dtype=torch.int32, device=gpu)
+    return q, k, v, cu_q, cu_k
+
+
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (16, 8), (8, 8)])
+def test_non_causal_sees_every_key(gpu, hq, hkv):
+    """causal=False: every query sees all sk keys of its sequence, also with more keys than queries.
+    Pinned twice: the oracle, and scaled_dot_product_attention without a mask on each sequence."""
+    lens_q, lens_k = [40, 1, 130, 64], [100, 33, 130, 700]
+    q, k, v, cu_q, cu_k = _packed_case(gpu, lens_q, lens_k, hq, hkv, seed=11)
+    scale = 0.11
+    out = ops.flash_attn_varlen_func(q, k, v, max_seqlen_q=max(lens_q), cu_seqlens_q=cu_q, max_seqlen_k=max(lens_k),
+                                     cu_seqlens_k=cu_k, softmax_scale=scale, causal=False)
+    want = paged_ref.varlen_prefill_ref(bits(q), bits(k), bits(v), cu_q.cpu().numpy(), cu_k.cpu().numpy(), scale,
+                                        causal=False)
+    assert np.abs(f32(out) - want).max() <= ATTN_ATOL
+    aq = ak = 0
+    for nq, nk in zip(lens_q, lens_k):
+        qq = q[aq:aq + nq].float().cpu().permute(1, 0, 2)
+        kk = k[ak:ak + nk].float().cpu().permute(1, 0, 2).repeat_interleave(hq // hkv, 0)
+        vv = v[ak:ak + nk].float().cpu().permute(1, 0, 2).repeat_interleave(hq // hkv, 0)
+        ref = torch.nn.functional.scaled_dot_product_attention(qq, kk, vv, scale=scale).permute(1, 0, 2)
+        assert (out[aq:aq + nq].float().cpu() - ref).abs().max() <= ATTN_ATOL
+        aq += nq
+        ak += nk
+
+
+def test_more_keys_than_queries_is_bottom_right_aligned(gpu):
+    """sq < sk with packed keys: query i sees keys 0 .. i + (sk - sq), the alignment the prefix-cache
+    branch relies on (infer/ops/attention.py:110-116)."""
+    lens_q, lens_k = [5, 64, 1], [37, 64, 300]
+    q, k, v, cu_q, cu_k = _packed_case(gpu, lens_q, lens_k, 16, 8, seed=12)
+    out = ops.flash_attn_varlen_func(q, k, v, max_seqlen_q=max(lens_q), cu_seqlens_q=cu_q, max_seqlen_k=max(lens_k),
+                                     cu_seqlens_k=cu_k, causal=True)
+    want = paged_ref.varlen_prefill_ref(bits(q), bits(k), bits(v), cu_q.cpu().numpy(), cu_k.cpu().numpy(), 128 ** -0.5)
+    assert np.abs(f32(out) - want).max() <= ATTN_ATOL
+    # the single query of the last sequence sees all 300 keys: one softmax row
+    s = (q[-1].float().cpu().view(8, 2, 128) @ k[-300:].float().cpu().permute(1, 2, 0)) * 128 ** -0.5
+    ref = torch.softmax(s, -1) @ v[-300:].float().cpu().permute(1, 0, 2)
+    assert (out[-1].float().cpu().view(8, 2, 128) - ref).abs().max() <= ATTN_ATOL
+
+
+@pytest.mark.parametrize("scale", [0.02, 0.25])
+def test_softmax_scale_is_honoured(gpu, scale):
+    wl = workloads.make_prefill_workload("p", [90, 300, 700], [0, 256, 512], 32, 8, seed=21, pad_fraction=0.0).to(gpu)
+    kc, vc = wl.k_cache.clone(), wl.v_cache.clone()
+    ops.store_kvcache(wl.k_new, wl.v_new, kc, vc, wl.slot_mapping)
+    out = ops.flash_attn_varlen_func(wl.q, kc, vc, max_seqlen_q=wl.max_seqlen_q, cu_seqlens_q=wl.cu_seqlens_q,
+                                     max_seqlen_k=wl.max_seqlen_k, cu_seqlens_k=wl.cu_seqlens_k,
+                                     softmax_scale=scale, causal=True, block_table=wl.block_table)
+    want = paged_ref.varlen_prefill_ref(bits(wl.q), bits(kc), bits(vc), wl.cu_seqlens_q.cpu().numpy(),
+                                        wl.cu_seqlens_k.cpu().numpy(), scale, block_table=wl.block_table.cpu().numpy())
+    assert np.abs(f32(out) - want).max() <= ATTN_ATOL
+
+
+def test_query_rows_as_views_of_the_qkv_projection(gpu):
+    """Q is a column slice of the fused qkv matrix in the reference (infer/models/Qwen3.py:110-111): its
+    rows are (Hq + 2 Hkv) * D apart.  Same bits as with a contiguous copy."""
+    wl = workloads.make_prefill_workload("p", [70, 513, 33], [0, 256, 0], 32, 8, seed=22, pad_fraction=0.0).to(gpu)
+    out, kc, vc = run_paged(wl)
+    t, hq, d = wl.q.shape
+    qkv = torch.randn((t, (hq + 16) * d), device=gpu).to(torch.bfloat16)
+    qkv[:, :hq * d] = wl.q.reshape(t, -1)
+    q_view = qkv.split([hq * d, 8 * d, 8 * d], dim=-1)[0].view(t, hq, d)
+    assert not q_view.is_contiguous()
+    out2 = ops.flash_attn_varlen_func(q_view, kc, vc, max_seqlen_q=wl.max_seqlen_q, cu_seqlens_q=wl.cu_seqlens_q,
+                                      max_seqlen_k=wl.max_seqlen_k, cu_seqlens_k=wl.cu_seqlens_k,
+                                      softmax_scale=wl.scale, causal=True, block_table=wl.block_table)
+    assert torch.equal(out, out2)
