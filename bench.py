@@ -207,10 +207,11 @@ def run_e2e(args):
 
 
 # ------------------------------------------------------------------------------------------ decode curve
-def decode_point(name, wl, copies, iters, splits=0):
+def decode_point(name, wl, copies, iters, splits=0, uniform_len=None):
     """Decode op (split + merge) of one workload, timed as replays of a HIP graph that holds ``copies``
     consecutive steps, each over its own copy of the caches (no host time between launches, reads
-    come from HBM)."""
+    come from HBM).  With ``uniform_len`` the batch's common length is also timed as a host integer
+    (``cache_seqlens: int``), the form in which the library may run one kernel without a merge."""
     from infer_amd import ops
     dev = wl.q.device
     b, hq, hkv, d = len(wl.lengths), wl.num_q_heads, wl.num_kv_heads, wl.head_dim
@@ -219,26 +220,36 @@ def decode_point(name, wl, copies, iters, splits=0):
     out = torch.empty((b, hq, d), dtype=torch.bfloat16, device=dev)
     ws = ops.decode_workspace(dev, b, hq, hkv, d)
 
-    def steps():
-        for i in range(copies):
-            ops.paged_attn_decode(wl.q, ks[i], vs[i], wl.block_table, wl.context_lens, wl.scale, out, ws,
-                                  split_workgroups=splits)
-    steps()
-    torch.cuda.synchronize()
-    side = torch.cuda.Stream()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.stream(side):
+    def timed(lengths):
+        def steps():
+            for i in range(copies):
+                ops.paged_attn_decode(wl.q, ks[i], vs[i], wl.block_table, lengths, wl.scale, out, ws,
+                                      split_workgroups=splits)
         steps()
-        side.synchronize()
-        with torch.cuda.graph(graph, stream=side):
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
             steps()
-    torch.cuda.synchronize()
-    ms = gpu_time_ms(graph.replay, iters, 2) / copies
+            side.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                steps()
+        torch.cuda.synchronize()
+        return gpu_time_ms(graph.replay, iters, 2) / copies
+
     nbytes = wl.decode_bytes
+
+    def figures(ms):
+        return {"op_us": round(ms * 1e3, 2), "GBps": round(nbytes / ms / 1e6, 1),
+                "frac_of_8TBps": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+
+    point = {"name": name, "batch": b, "Hq": hq, "tokens": sum(wl.lengths), "algorithmic_bytes": nbytes,
+             **figures(timed(wl.context_lens)), "cache_copies": copies}
+    if uniform_len is not None:
+        assert all(n == uniform_len for n in wl.lengths)
+        point["length_as_host_int"] = figures(timed(int(uniform_len)))
     del ks, vs
-    return {"name": name, "batch": b, "Hq": hq, "tokens": sum(wl.lengths), "algorithmic_bytes": nbytes,
-            "op_us": round(ms * 1e3, 2), "GBps": round(nbytes / ms / 1e6, 1),
-            "frac_of_8TBps": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "cache_copies": copies}
+    return point
 
 
 def decode_curve(dev, iters=12):
@@ -251,7 +262,8 @@ def decode_curve(dev, iters=12):
         wl = workloads.make_decode_workload(f"b64-ctx{ctx}", [ctx] * 64, 32, 8, seed=ctx, q_scale=128 ** -0.5,
                                             device=dev, device_fill=True)
         pool_mb = 2 * wl.k_cache.numel() * 2 / 1e6
-        points.append(decode_point(f"batch 64 x ctx {ctx}", wl, max(2, min(8, int(1100 / pool_mb) + 1)), iters))
+        points.append(decode_point(f"batch 64 x ctx {ctx}", wl, max(2, min(8, int(1100 / pool_mb) + 1)), iters,
+                                   uniform_len=ctx))
         del wl
         torch.cuda.empty_cache()
     gen = torch.Generator().manual_seed(5)
@@ -262,7 +274,7 @@ def decode_curve(dev, iters=12):
     del wl
     torch.cuda.empty_cache()
     wl = workloads.cfg4(device=dev, device_fill=True)
-    points.append(decode_point("cfg4: batch 8 x ctx 32768, Hq=64", wl, 2, iters))
+    points.append(decode_point("cfg4: batch 8 x ctx 32768, Hq=64", wl, 2, iters, uniform_len=32768))
     del wl
     torch.cuda.empty_cache()
     return points

@@ -172,6 +172,28 @@ int infer_paged_decode_merge_bf16(void* out, int64_t out_stride0,
                                   const void* workspace, size_t workspace_bytes,
                                   void* stream);
 
+/* The decode call with the context length given as ONE host integer for the whole batch, the
+ * `cache_seqlens: int` form of flash_attn_with_kvcache (the function called at
+ * infer/ops/attention.py:118-120; the reference itself passes the per-sequence tensor).  Same result
+ * as infer_paged_decode_bf16 with context_lens[b] == context_len for every b; context_len == 0
+ * gives zeros.  Knowing the length on the host, the library needs no span plan: when batch x KV
+ * heads fills the chip with whole workgroups per sequence (batch x num_kv_heads x p / 8 within
+ * 80 - 100 % of the compute units for a p in {1, 2, 4, 8}), one kernel streams each sequence in p
+ * pieces per KV head, folds them in LDS and writes the result, with no partial results in memory and
+ * no merge launch; other shapes run the two kernels of infer_paged_decode_bf16 without reading a
+ * lengths array.  The workspace is the one of infer_paged_decode_bf16 (used by the second case). */
+int infer_paged_decode_uniform_bf16(const void* q, int64_t q_stride0,
+                                    const void* k_cache, const void* v_cache,
+                                    int64_t cache_block_stride, int64_t cache_token_stride,
+                                    void* out, int64_t out_stride0,
+                                    const int32_t* block_table, int64_t bt_stride0, int64_t table_cols,
+                                    int64_t context_len,
+                                    int64_t batch, int64_t num_q_heads, int64_t num_kv_heads,
+                                    int64_t head_dim, int64_t block_size, int64_t num_blocks,
+                                    float scale,
+                                    void* workspace, size_t workspace_bytes,
+                                    void* stream);
+
 /* infer_paged_decode_bf16 for callers that cannot allocate and have no workspace to bring: code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in
  * the reference.  Same arguments, result and kernels as infer_paged_decode_bf16 with

@@ -34,6 +34,8 @@ SIGNATURES = {
                                                  _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _vp, _sz, _vp]),
     "infer_paged_decode_noalloc_bf16": (_c.c_int, [_vp, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _vp,
                                                    _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp]),
+    "infer_paged_decode_uniform_bf16": (_c.c_int, [_vp, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _i64,
+                                                   _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp, _sz, _vp]),
     "infer_paged_decode_merge_bf16": (_c.c_int, [_vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _sz, _vp]),
     "infer_paged_prefill_bf16": (_c.c_int, [_vp, _i64, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _i64,
                                             _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _c.c_int, _vp]),

@@ -197,7 +197,7 @@ int infer_kv_append_bf16(const void* key, int64_t key_stride0, const void* value
     return (int)hipGetLastError();
 }
 
-const char* infer_kv_version(void) { return "0.2"; }
+const char* infer_kv_version(void) { return "0.3"; }
 
 const char* infer_kv_strerror(int code) {
     switch (code) {

@@ -55,7 +55,8 @@ struct DecodeArgs {
     int64_t tok_stride;
     const int32_t* bt;
     int64_t bt_stride0;
-    const int32_t* ctx;
+    const int32_t* ctx; // nullptr: every sequence has uniform_len tokens
+    int uniform_len;
     int max_ctx;        // lengths are clamped to what the block table can address (table_cols * block_size)
     int batch;
     int group;          // query heads per KV head
@@ -69,6 +70,8 @@ struct DecodeArgs {
     unsigned char* rec; // [slots] partial-result records (layout: decode_record_bytes)
     int rec_stride;
     int slots_per_head; // records per KV head in the workspace (layout constant, >= gridDim.x + batch)
+    uint16_t* out;      // uniform kernel only: it writes the result itself
+    int64_t out_stride0;
 };
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 x) { return __builtin_bit_cast(bf16x8, x); }
@@ -89,9 +92,9 @@ __device__ __forceinline__ int steps_of(int len) { return len > 0 ? (len + kStep
 
 // Context length of sequence i as the kernels use it: a length the block table row cannot address is
 // cut to the row's capacity, so a corrupt length cannot make the table gather run past the row.
-__device__ __forceinline__ int ctx_len(const int32_t* ctx, int max_ctx, int i) {
-    const int len = ctx[i];
-    return len < max_ctx ? len : max_ctx;
+__device__ __forceinline__ int ctx_len(const DecodeArgs& a, int i) {
+    const int len = a.ctx ? a.ctx[i] : a.uniform_len;
+    return len < a.max_ctx ? len : a.max_ctx;
 }
 
 // Inclusive prefix sum over the 64 lanes on the vector pipe (data-parallel primitives): shifts by 1,
@@ -196,6 +199,7 @@ struct StepCursor {
 // then K(i+2) and V(i+1) are in flight, across sequence boundaries.  Loads past the end of the
 // batch are redirected to one dummy 16-byte location instead of being skipped, which keeps the
 // number of outstanding loads at every wait independent of control flow.
+template <bool kKeep = false>
 __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* lds, const int* plan, int nseg,
                                           int total_steps, int tblv_loaded, int h, int w, int lane) {
     // The block ids were gathered by vector loads.  Hand them to the loop as a plain register value:
@@ -433,7 +437,79 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
     }
     if (i < total_steps) step(P0{});
     lds_order();
-    drain();
+    if (!kKeep) drain();   // kKeep: a single segment whose partial result stays parked in LDS for the caller
+}
+
+// Uniform batch: every sequence has the same number of tokens, known on the host.  A workgroup is
+// 8 wavefronts = (8 / parts) KV heads of ONE sequence x `parts` pieces of its steps.  The pieces of a
+// head are folded through LDS and the workgroup writes the bf16 result itself: no span plan (the
+// block ids are the only load in front of the first K row), no partial result in memory, no merge
+// launch.  The price is that a workgroup reads (8 / parts) x 256 B of every token row instead of
+// the whole 2 KiB row.
+__global__ void __launch_bounds__(512) paged_decode_uniform_kernel(DecodeArgs a, int parts) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_all[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int heads_per_wg = 8 / parts;
+    const int wg_per_seq = a.num_kv_heads / heads_per_wg;
+    const int b = blockIdx.x / wg_per_seq;
+    const int h = (blockIdx.x % wg_per_seq) * heads_per_wg + wave / parts;   // consecutive wavefronts: the pieces of one head
+    const int part = wave % parts;
+    unsigned char* lds = lds_all + wave * kLdsPerWave;
+    int* plan = reinterpret_cast<int*>(lds + kLdsWave);
+    unsigned char* defer = lds + kLdsWave + kPlanBytes;
+    const int steps_per_blk = a.block_size / kStep;
+    const int G = a.group;
+    const int g = lane >> 4, n = lane & 15;
+    const int len = a.uniform_len < a.max_ctx ? a.uniform_len : a.max_ctx;
+    const int nsteps = steps_of(len), share = (nsteps + parts - 1) / parts;
+    const int s_lo = part * share, s_hi = s_lo + share < nsteps ? s_lo + share : nsteps;
+    if (s_lo < s_hi) {
+        const int blk0 = s_lo / steps_per_blk;
+        const int nblk = (s_hi - 1) / steps_per_blk - blk0 + 1;
+        if (lane == 0) {
+            plan[0] = b; plan[1] = len; plan[2] = s_lo; plan[3] = s_hi; plan[4] = 0;
+            plan[5] = s_lo - blk0 * steps_per_blk; plan[6] = blk0;
+        }
+        int tblv = 0;   // lane i = i-th block of this piece (a piece of more than 64 blocks looks the rest up)
+        if (lane < nblk) tblv = a.bt[(int64_t)b * a.bt_stride0 + blk0 + lane];
+        lds_order();
+        run_batch<true>(a, lds, plan, 1, s_hi - s_lo, tblv, h, 0, lane);
+    } else if (g == 0 && n < G) {
+        // fewer steps than pieces: an empty piece parks an empty (max, sum)
+        *reinterpret_cast<float2*>(defer + 512 * G + n * 8) = make_float2(-INFINITY, 0.f);
+    }
+    __syncthreads();
+    if (part != 0 || n >= G) return;
+    // piece 0 of every head folds the records of its `parts` pieces (the next wavefronts' LDS areas);
+    // lane (g, n) holds head n, columns 16 t + 4 g .. + 3 of accumulator tile t
+    const int vlane = g * G + n;
+    float m = -INFINITY;
+    for (int p = 0; p < parts; ++p)
+        m = fmaxf(m, reinterpret_cast<const float2*>(defer + p * kLdsPerWave + 512 * G + n * 8)->x);
+    float den = 0.f;
+    f32x4 num[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) num[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int p = 0; p < parts; ++p) {
+        const unsigned char* r = defer + p * kLdsPerWave;
+        const float2 ml = *reinterpret_cast<const float2*>(r + 512 * G + n * 8);
+        if (ml.y > 0.f) {
+            const float f = __builtin_amdgcn_exp2f(ml.x - m);
+            den += ml.y * f;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) num[t] += *reinterpret_cast<const f32x4*>(r + (vlane * 8 + t) * 16) * f;
+        }
+    }
+    const float inv = den > 0.f ? 1.f / den : 0.f;
+    uint16_t* op = a.out + (int64_t)b * a.out_stride0 + (int64_t)(h * G + n) * kD + 4 * g;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        union { __bf16 hv[4]; u32x2 u; } r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r.hv[e] = (__bf16)(num[t][e] * inv);
+        *reinterpret_cast<u32x2*>(op + 16 * t) = r.u;
+    }
 }
 
 __global__ void __launch_bounds__(512) paged_decode_split_kernel(DecodeArgs a) {
@@ -449,11 +525,11 @@ __global__ void __launch_bounds__(512) paged_decode_split_kernel(DecodeArgs a) {
     const int steps_per_blk = a.block_size / kStep;
 
     // total number of steps (the first 64 lengths stay in registers for the second pass)
-    const int len0 = lane < a.batch ? ctx_len(a.ctx, a.max_ctx, lane) : 0;
+    const int len0 = lane < a.batch ? ctx_len(a, lane) : 0;
     int total = wave_sum(steps_of(len0));
     for (int c = 64; c < a.batch; c += 64) {
         const int i = c + lane;
-        total += wave_sum(i < a.batch ? steps_of(ctx_len(a.ctx, a.max_ctx, i)) : 0);
+        total += wave_sum(i < a.batch ? steps_of(ctx_len(a, i)) : 0);
     }
     total = __builtin_amdgcn_readfirstlane(total);   // wave-uniform: keep the plan in scalar registers
 
@@ -486,7 +562,7 @@ __global__ void __launch_bounds__(512) paged_decode_split_kernel(DecodeArgs a) {
     int running = 0;
     for (int c = 0; c < a.batch; c += 64) {
         const int i = c + lane;
-        const int len = c == 0 ? len0 : (i < a.batch ? ctx_len(a.ctx, a.max_ctx, i) : 0);
+        const int len = c == 0 ? len0 : (i < a.batch ? ctx_len(a, i) : 0);
         const int cnt = steps_of(len);
         const int incl = wave_inclusive_scan(cnt, lane);
         const int start = running + incl - cnt;
@@ -538,7 +614,8 @@ __global__ void __launch_bounds__(512) paged_decode_split_kernel(DecodeArgs a) {
 struct MergeArgs {
     uint16_t* out;
     int64_t out_stride0;
-    const int32_t* ctx;
+    const int32_t* ctx;     // nullptr: every sequence has uniform_len tokens
+    int uniform_len;
     int group;
     int slots_per_head;     // records per KV head in the workspace, as in the split launch
     const int32_t* seg_first;
@@ -560,7 +637,7 @@ __global__ void __launch_bounds__(256) paged_decode_merge_kernel(MergeArgs a) {
     const int h = head / G, n = head - h * G;
     const int j = threadIdx.x >> 5, c4 = threadIdx.x & 31;
     uint16_t* op = a.out + (int64_t)b * a.out_stride0 + (int64_t)head * kD + 4 * c4;
-    if (a.ctx[b] <= 0) {
+    if ((a.ctx ? a.ctx[b] : a.uniform_len) <= 0) {
         if (j == 0) *reinterpret_cast<u32x2*>(op) = u32x2{0u, 0u};
         return;
     }
@@ -677,14 +754,15 @@ struct DecodeCall {
     const void* k_cache; const void* v_cache;
     int64_t cache_block_stride, cache_token_stride;
     const int32_t* block_table; int64_t bt_stride0, table_cols;
-    const int32_t* context_lens;
+    const int32_t* context_lens;   // nullptr: every sequence has uniform_len tokens
     int64_t batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks;
     float scale;
+    int64_t uniform_len = 0;
 };
 
 // Checks every argument of the split phase and fills in the launch shape.
 int check_split(const DecodeCall& c, int64_t split_workgroups, const void* workspace, Launch* L) {
-    if (!c.q || !c.k_cache || !c.v_cache || !c.block_table || !c.context_lens || !workspace) return INFER_KV_EINVAL;
+    if (!c.q || !c.k_cache || !c.v_cache || !c.block_table || !workspace) return INFER_KV_EINVAL;
     int rc = check_shape(c.batch, c.num_q_heads, c.num_kv_heads, c.head_dim, c.block_size, c.num_blocks, c.table_cols);
     if (rc) return rc;
     // 16-byte vector loads: every row start must be 16-byte aligned.
@@ -717,6 +795,9 @@ int launch_split(const DecodeCall& c, const Launch& L, const DecodeWorkspace& ws
     a.bt = c.block_table;
     a.bt_stride0 = c.bt_stride0;
     a.ctx = c.context_lens;
+    a.uniform_len = c.uniform_len > 0x7fffffffLL ? 0x7fffffff : (c.uniform_len < 0 ? 0 : (int)c.uniform_len);
+    a.out = nullptr;
+    a.out_stride0 = 0;
     const int64_t max_ctx = c.table_cols * c.block_size;
     a.max_ctx = max_ctx > 0x7fffffffLL ? 0x7fffffff : (int)max_ctx;
     a.batch = (int)c.batch;
@@ -747,13 +828,71 @@ int launch_split(const DecodeCall& c, const Launch& L, const DecodeWorkspace& ws
     return (int)hipGetLastError();
 }
 
-int launch_merge(void* out, int64_t out_stride0, const int32_t* context_lens, int64_t batch, int64_t num_q_heads,
-                 int64_t num_kv_heads, const DecodeWorkspace& ws, const void* base_v, hipStream_t stream) {
+// Pieces per KV head for the uniform kernel, or 0 when the span kernel serves the shape better.  The
+// uniform kernel holds one 8-wavefront workgroup per compute unit (its LDS), so it is used when
+// batch x KV heads x pieces / 8 workgroups fill the chip in one round with even pieces.
+int uniform_parts(const DecodeCall& c) {
+    if (c.uniform_len <= 0 || c.num_kv_heads > (1 << 16)) return 0;
+    const int64_t cus = device_cu_count();
+    const int64_t len = c.uniform_len < c.table_cols * c.block_size ? c.uniform_len : c.table_cols * c.block_size;
+    const int64_t steps = (len + kStep - 1) / kStep;
+    for (int parts = 8; parts >= 1; parts >>= 1) {
+        const int heads_per_wg = 8 / parts;
+        if (c.num_kv_heads % heads_per_wg != 0) continue;
+        const int64_t wgs = c.batch * (c.num_kv_heads / heads_per_wg);
+        if (wgs > cus) continue;
+        if (wgs * 5 < cus * 4) return 0;                        // the largest fit leaves a fifth of the chip idle
+        const int64_t share = (steps + parts - 1) / parts;
+        return steps * 20 >= share * parts * 17 ? parts : 0;    // pieces at least 85 % even
+    }
+    return 0;
+}
+
+int launch_uniform(const DecodeCall& c, void* out, int64_t out_stride0, int parts, hipStream_t stream) {
+    DecodeArgs a{};
+    a.q = (const uint16_t*)c.q;
+    a.q_stride0 = c.q_stride0;
+    a.k = (const uint16_t*)c.k_cache;
+    a.v = (const uint16_t*)c.v_cache;
+    a.blk_stride = c.cache_block_stride;
+    a.tok_stride = c.cache_token_stride;
+    a.bt = c.block_table;
+    a.bt_stride0 = c.bt_stride0;
+    a.ctx = nullptr;
+    a.uniform_len = c.uniform_len > 0x7fffffffLL ? 0x7fffffff : (int)c.uniform_len;
+    const int64_t max_ctx = c.table_cols * c.block_size;
+    a.max_ctx = max_ctx > 0x7fffffffLL ? 0x7fffffff : (int)max_ctx;
+    a.batch = (int)c.batch;
+    a.group = (int)(c.num_q_heads / c.num_kv_heads);
+    a.num_kv_heads = (int)c.num_kv_heads;
+    a.block_size = (int)c.block_size;
+    a.num_blocks = (int)c.num_blocks;
+    a.scale_log2 = c.scale * 1.4426950408889634f;
+    a.rec_stride = (int)decode_record_bytes(a.group);   // layout of a parked partial result
+    a.out = (uint16_t*)out;
+    a.out_stride0 = out_stride0;
+    static bool attr_set[kMaxDevices] = {false};   // the attribute is per device
+    const int dev = current_device();
+    if (!attr_set[dev]) {
+        hipError_t e = hipFuncSetAttribute((const void*)paged_decode_uniform_kernel,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 8 * kLdsPerWave);
+        if (e != hipSuccess) return (int)e;
+        attr_set[dev] = true;
+    }
+    const unsigned wgs = (unsigned)(c.batch * (c.num_kv_heads / (8 / parts)));
+    hipLaunchKernelGGL(paged_decode_uniform_kernel, dim3(wgs, 1, 1), dim3(512, 1, 1), 8 * kLdsPerWave, stream, a, parts);
+    return (int)hipGetLastError();
+}
+
+int launch_merge(void* out, int64_t out_stride0, const int32_t* context_lens, int64_t uniform_len, int64_t batch,
+                 int64_t num_q_heads, int64_t num_kv_heads, const DecodeWorkspace& ws, const void* base_v,
+                 hipStream_t stream) {
     const char* base = (const char*)base_v;
     MergeArgs m;
     m.out = (uint16_t*)out;
     m.out_stride0 = out_stride0;
     m.ctx = context_lens;
+    m.uniform_len = uniform_len > 0 ? 1 : 0;   // only its sign matters here
     m.group = (int)(num_q_heads / num_kv_heads);
     m.slots_per_head = (int)ws.slots_per_head;
     m.seg_first = (const int32_t*)(base + ws.seg_first_off);
@@ -818,6 +957,7 @@ int infer_paged_decode_split_bf16(const void* q, int64_t q_stride0, const void* 
     const DecodeCall c{q, q_stride0, k_cache, v_cache, cache_block_stride, cache_token_stride, block_table, bt_stride0,
                        table_cols, context_lens, batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks,
                        scale};
+    if (!context_lens) return INFER_KV_EINVAL;
     Launch L;
     int rc = check_split(c, split_workgroups, workspace, &L);
     if (rc) return rc;
@@ -838,7 +978,7 @@ int infer_paged_decode_merge_bf16(void* out, int64_t out_stride0, const int32_t*
     if ((uintptr_t)workspace & 15) return INFER_KV_EALIGN;   // 16-byte loads of the records
     const DecodeWorkspace ws = decode_workspace_layout(batch, num_q_heads / num_kv_heads, num_kv_heads);
     if (ws.total_bytes > workspace_bytes) return INFER_KV_EWORKSPACE;
-    return launch_merge(out, out_stride0, context_lens, batch, num_q_heads, num_kv_heads, ws, workspace,
+    return launch_merge(out, out_stride0, context_lens, 0, batch, num_q_heads, num_kv_heads, ws, workspace,
                         (hipStream_t)stream);
 }
 
@@ -853,6 +993,7 @@ int infer_paged_decode_bf16(const void* q, int64_t q_stride0, const void* k_cach
                        table_cols, context_lens, batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks,
                        scale};
     // everything is checked before the first launch is enqueued
+    if (!context_lens) return INFER_KV_EINVAL;
     Launch L;
     int rc = check_split(c, split_workgroups, workspace, &L);
     if (rc) return rc;
@@ -862,7 +1003,32 @@ int infer_paged_decode_bf16(const void* q, int64_t q_stride0, const void* k_cach
     if (ws.total_bytes > workspace_bytes) return INFER_KV_EWORKSPACE;
     rc = launch_split(c, L, ws, workspace, (hipStream_t)stream);
     if (rc) return rc;
-    return launch_merge(out, out_stride0, context_lens, batch, num_q_heads, num_kv_heads, ws, workspace,
+    return launch_merge(out, out_stride0, context_lens, 0, batch, num_q_heads, num_kv_heads, ws, workspace,
+                        (hipStream_t)stream);
+}
+
+int infer_paged_decode_uniform_bf16(const void* q, int64_t q_stride0, const void* k_cache, const void* v_cache,
+                                    int64_t cache_block_stride, int64_t cache_token_stride, void* out,
+                                    int64_t out_stride0, const int32_t* block_table, int64_t bt_stride0,
+                                    int64_t table_cols, int64_t context_len, int64_t batch, int64_t num_q_heads,
+                                    int64_t num_kv_heads, int64_t head_dim, int64_t block_size, int64_t num_blocks,
+                                    float scale, void* workspace, size_t workspace_bytes, void* stream) {
+    DecodeCall c{q, q_stride0, k_cache, v_cache, cache_block_stride, cache_token_stride, block_table, bt_stride0,
+                 table_cols, nullptr, batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, scale};
+    c.uniform_len = context_len;
+    if (context_len < 0 || context_len > 0x7fffffffLL) return INFER_KV_EINVAL;
+    Launch L;
+    int rc = check_split(c, /*split_workgroups=*/0, workspace, &L);
+    if (rc) return rc;
+    rc = check_out(out, out_stride0, num_q_heads);
+    if (rc) return rc;
+    const DecodeWorkspace ws = decode_workspace_layout(batch, num_q_heads / num_kv_heads, num_kv_heads);
+    if (ws.total_bytes > workspace_bytes) return INFER_KV_EWORKSPACE;
+    if (const int parts = uniform_parts(c)) return launch_uniform(c, out, out_stride0, parts, (hipStream_t)stream);
+    // shapes the uniform kernel does not fill the chip with: equal spans + merge, without a lengths array
+    rc = launch_split(c, L, ws, workspace, (hipStream_t)stream);
+    if (rc) return rc;
+    return launch_merge(out, out_stride0, nullptr, context_len, batch, num_q_heads, num_kv_heads, ws, workspace,
                         (hipStream_t)stream);
 }
 
@@ -875,6 +1041,7 @@ int infer_paged_decode_noalloc_bf16(const void* q, int64_t q_stride0, const void
     const DecodeCall c{q, q_stride0, k_cache, v_cache, cache_block_stride, cache_token_stride, block_table, bt_stride0,
                        table_cols, context_lens, batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks,
                        scale};
+    if (!context_lens) return INFER_KV_EINVAL;
     void* scratch = nullptr;
     int rc = noalloc_scratch(&scratch);
     if (rc) return rc;
@@ -888,7 +1055,7 @@ int infer_paged_decode_noalloc_bf16(const void* q, int64_t q_stride0, const void
     if (ws.total_bytes > kNoAllocScratchBytes) return INFER_KV_EWORKSPACE;
     rc = launch_split(c, L, ws, scratch, (hipStream_t)stream);
     if (rc) return rc;
-    return launch_merge(out, out_stride0, context_lens, batch, num_q_heads, num_kv_heads, ws, scratch,
+    return launch_merge(out, out_stride0, context_lens, 0, batch, num_q_heads, num_kv_heads, ws, scratch,
                         (hipStream_t)stream);
 }
 

@@ -127,17 +127,18 @@ def decode_workspace(device, max_batch: int, num_q_heads: int, num_kv_heads: int
 
 def _decode_args(q3, k_cache, v_cache, cache_seqlens, block_table):
     assert q3.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16
-    assert cache_seqlens.dtype == torch.int32 and block_table.dtype == torch.int32
+    uniform = isinstance(cache_seqlens, int)      # one length for the whole batch, known on the host
+    assert block_table.dtype == torch.int32 and (uniform or cache_seqlens.dtype == torch.int32)
     assert k_cache.dim() == 4 and k_cache.shape == v_cache.shape
     assert k_cache.stride() == v_cache.stride()
     b, hq, d = q3.shape
     nblk, bs, hkv, dk = k_cache.shape
     assert dk == d and q3.stride(2) == 1 and q3.stride(1) == d
     assert k_cache.stride(3) == 1 and k_cache.stride(2) == d
-    assert cache_seqlens.numel() == b and cache_seqlens.is_contiguous()
+    assert cache_seqlens >= 0 if uniform else (cache_seqlens.numel() == b and cache_seqlens.is_contiguous())
     assert block_table.dim() == 2 and block_table.shape[0] == b and block_table.shape[1] >= 1
     assert block_table.stride(1) == 1
-    _require_gpu(q3, k_cache, v_cache, cache_seqlens, block_table)
+    _require_gpu(q3, k_cache, v_cache, block_table, *(() if uniform else (cache_seqlens,)))
     return b, hq, d, nblk, bs, hkv
 
 
@@ -147,12 +148,25 @@ def paged_attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     """Out-parameter form: ``q``/``out`` are ``[B, Hq, D]``.  ``split_workgroups`` = workgroups along
     the KV-split axis of this call (0: the library's choice for the device).  The default workspace is
     shared by every call for the shape on the device, so such calls must be ordered on one stream;
-    pass a ``workspace`` of its own to a call that runs on another stream."""
+    pass a ``workspace`` of its own to a call that runs on another stream.
+
+    ``context_lens`` is the int32 tensor of the reference's call, or a Python int when every sequence
+    of the batch has that many tokens (``cache_seqlens: int`` of ``flash_attn_with_kvcache``): the
+    library then plans the launch on the host and, for batches that fill the chip, runs one kernel
+    without a merge launch (``split_workgroups`` does not apply)."""
     b, hq, d, nblk, bs, hkv = _decode_args(q, k_cache, v_cache, context_lens, block_table)
     assert out.shape == q.shape and out.dtype == torch.bfloat16 and out.stride(2) == 1 and out.stride(1) == d
     if workspace is None:
         workspace = decode_workspace(q.device, b, hq, hkv, d)
     lib = _lib.load()
+    if isinstance(context_lens, int):
+        rc = lib.infer_paged_decode_uniform_bf16(
+            q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), k_cache.stride(0), k_cache.stride(1),
+            out.data_ptr(), out.stride(0), block_table.data_ptr(), block_table.stride(0), block_table.shape[1],
+            context_lens, b, hq, hkv, d, bs, nblk, float(scale), workspace.data_ptr(), workspace.numel(),
+            _stream_ptr(q))
+        _lib.check(rc, "paged_attn_decode")
+        return
     rc = lib.infer_paged_decode_bf16(
         q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), k_cache.stride(0), k_cache.stride(1),
         out.data_ptr(), out.stride(0), block_table.data_ptr(), block_table.stride(0), block_table.shape[1],
@@ -182,10 +196,11 @@ def paged_attn_decode_merge(out, context_lens, num_kv_heads, workspace) -> None:
 
 
 def flash_attn_with_kvcache(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, *,
-                            cache_seqlens: torch.Tensor, block_table: torch.Tensor,
+                            cache_seqlens: "torch.Tensor | int", block_table: torch.Tensor,
                             softmax_scale: float | None = None, causal: bool = True) -> torch.Tensor:
     """``q`` is ``[B, 1, Hq, D]``; returns ``[B, 1, Hq, D]``.  With a single query token the causal
-    mask hides nothing, so ``causal`` only has to be accepted."""
+    mask hides nothing, so ``causal`` only has to be accepted.  ``cache_seqlens`` is an int32 tensor
+    ``[B]`` or one int for the whole batch, as in flash-attn."""
     assert q.dim() == 4 and q.shape[1] == 1, "decode takes one query token per sequence"
     if softmax_scale is None:
         softmax_scale = q.shape[-1] ** -0.5

@@ -48,7 +48,7 @@ def test_library_exports_every_declared_symbol_and_binding_covers_it():
 
 def test_host_only_entry_points():
     lib = _lib.load()
-    assert lib.infer_kv_version() == b"0.2"
+    assert lib.infer_kv_version() == b"0.3"
     assert b"workspace" in lib.infer_kv_strerror(-3)
     assert lib.infer_paged_decode_workspace_bytes(64, 32, 8, 128) > 0
     assert lib.infer_paged_decode_workspace_bytes(64, 32, 8, 64) == 0        # head_dim not built
@@ -87,6 +87,18 @@ def test_argument_errors_are_reported_before_anything_is_launched():
                                        2, 32, 8, 128, 256, 4, 1.0, -1, p16, 1 << 30, None) == -1
     assert lib.infer_paged_decode_bf16(p16, 4096, p16, p16, 262144, 1024, p16, 4096, p16, 1 << 23, 1 << 23, p16,
                                        1 << 10, 32, 8, 128, 256, 4, 1.0, 0, p16, 1 << 40, None) == -1
+    # the lengths array is required where it is an argument; the uniform form takes a non-negative length,
+    # an output it can store to and a workspace for the shapes that need one
+    assert lib.infer_paged_decode_bf16(p16, 4096, p16, p16, 262144, 1024, p16, 4096, p16, 4, 4, None,
+                                       2, 32, 8, 128, 256, 4, 1.0, 0, p16, 1 << 30, None) == -1
+    assert lib.infer_paged_decode_uniform_bf16(p16, 4096, p16, p16, 262144, 1024, p16, 4096, p16, 4, 4, -1,
+                                               2, 32, 8, 128, 256, 4, 1.0, p16, 1 << 30, None) == -1
+    assert lib.infer_paged_decode_uniform_bf16(p16, 4096, p16, p16, 262144, 1024, p16 + 2, 4096, p16, 4, 4, 100,
+                                               2, 32, 8, 128, 256, 4, 1.0, p16, 1 << 30, None) == -2
+    assert lib.infer_paged_decode_uniform_bf16(p16, 4096, p16, p16, 262144, 1024, p16, 4096, p16, 4, 4, 100,
+                                               2, 32, 8, 128, 256, 4, 1.0, p16, 64, None) == -3
+    assert lib.infer_paged_decode_uniform_bf16(p16, 4096, p16, p16, 262144, 1024, p16, 4096, p16, 4, 4, 100,
+                                               2, 32, 8, 64, 256, 4, 1.0, p16, 1 << 30, None) == -4   # head_dim
     # prefill: the scale must be positive (the row maximum is taken before scaling)
     for bad_scale in (0.0, -0.1, float("nan")):
         assert lib.infer_paged_prefill_bf16(p16, 4096, p16, p16, 262144, 1024, 1024, p16, 4096, p16, p16, p16, 4, 4,

@@ -360,3 +360,86 @@ def test_query_and_output_rows_as_strided_views(gpu):
     torch.cuda.synchronize()
     assert torch.equal(out_view, want)
     assert (wide[:, hq * d:] == 7.0).all()      # nothing written beside the output rows
+
+
+def uniform_decode(wl, length):
+    out = torch.full_like(wl.q, 7.0)
+    ops.paged_attn_decode(wl.q, wl.k_cache, wl.v_cache, wl.block_table, length, wl.scale, out)
+    torch.cuda.synchronize()
+    return out
+
+
+# batch, context length, Hq, Hkv: shapes on both sides of the rule that picks the one-kernel form
+# (batch x Hkv x pieces / 8 workgroups within 80-100 % of the compute units, even pieces)
+UNIFORM_SHAPES = [
+    (64, 512, 32, 8),     # 4 pieces per KV head
+    (64, 517, 64, 8),     # ... a ragged last step, group size 8
+    (128, 300, 32, 8),    # 2 pieces
+    (32, 1000, 16, 8),    # 8 pieces: one KV head per workgroup
+    (256, 100, 8, 8),     # 1 piece: a sequence per workgroup, nothing to fold
+    (240, 65, 16, 8),     # 240 of 256 workgroups
+    (128, 130, 128, 16),  # 16 KV heads, group size 8
+    (256, 128, 8, 2),     # 2 KV heads: 4 pieces
+    (64, 33, 32, 8),      # fewer steps than pieces: span kernels without a lengths array
+    (4, 700, 16, 8),      # too few sequences to fill the chip: span kernels
+    (100, 260, 32, 8),    # 100 or 200 workgroups: span kernels
+    (3, 1, 16, 8),
+]
+
+
+@pytest.mark.parametrize("batch,length,hq,hkv", UNIFORM_SHAPES)
+def test_one_length_for_the_batch_as_a_host_integer(gpu, batch, length, hq, hkv):
+    """cache_seqlens given as one int (flash_attn_with_kvcache accepts both): same result as the tensor
+    form, against the oracle, whichever kernels the library picks for the shape."""
+    wl = workloads.make_decode_workload("uniform", [length] * batch, hq, hkv, seed=batch + length).to(gpu)
+    got = uniform_decode(wl, length)
+    want = oracle_decode(wl)
+    assert np.isfinite(f32(got)).all()
+    assert np.abs(f32(got) - want).max() <= ATTN_ATOL
+    # the tensor form folds the same partial sums in another order: two bf16 roundings of close fp32 values
+    assert (got.float() - gpu_decode(wl, splits=0).float()).abs().max() <= 8e-3
+    via_flash = ops.flash_attn_with_kvcache(wl.q.unsqueeze(1), wl.k_cache, wl.v_cache, cache_seqlens=length,
+                                            block_table=wl.block_table, softmax_scale=wl.scale)[:, 0]
+    assert torch.equal(via_flash, got)
+
+
+def test_uniform_length_edge_cases(gpu):
+    wl = workloads.make_decode_workload("uniform-edges", [300] * 64, 32, 8, seed=77).to(gpu)
+    assert (uniform_decode(wl, 0) == 0).all()                       # no context: zeros, as the tensor form
+    # one token: softmax over one key is 1, the output is that token's V row for every head of the group
+    one = uniform_decode(wl, 1)
+    v_first = wl.v_cache[wl.block_table[:, 0].long(), 0]            # [B, Hkv, D]
+    assert torch.equal(one, v_first.repeat_interleave(4, dim=1))
+    # a length the table row cannot address is cut to the row: 2 columns x 256 tokens
+    cut = uniform_decode(wl, 10_000)
+    wl2 = workloads.make_decode_workload("uniform-edges", [300] * 64, 32, 8, seed=77).to(gpu)
+    wl2.context_lens[:] = wl2.block_table.shape[1] * 256
+    # the table rows address 512 tokens: the same as asking for 512, in either form
+    assert torch.equal(cut, uniform_decode(wl, wl.block_table.shape[1] * 256))
+    assert (cut.float() - gpu_decode(wl2, splits=0).float()).abs().max() <= 8e-3
+    # stale NaN behind the length is never read into the result
+    for i in range(64):
+        blk = int(wl.block_table[i, 1])
+        wl.k_cache[blk, 300 % 256:] = float("nan")
+        wl.v_cache[blk, 300 % 256:] = float("nan")
+    got = uniform_decode(wl, 300)
+    assert np.isfinite(f32(got)).all()
+    keep = wl.context_lens.clone()
+    assert np.abs(f32(got) - oracle_decode(wl)).max() <= ATTN_ATOL and torch.equal(keep, wl.context_lens)
+
+
+def test_uniform_form_on_strided_views_and_other_block_sizes(gpu):
+    for bs in (32, 64, 512):
+        wl = workloads.make_decode_workload("uniform-bs", [2 * bs + 5] * 64, 32, 8, bs=bs, seed=bs).to(gpu)
+        assert np.abs(f32(uniform_decode(wl, 2 * bs + 5)) - oracle_decode(wl)).max() <= ATTN_ATOL
+    wl = workloads.make_decode_workload("uniform-views", [400] * 64, 32, 8, seed=5).to(gpu)
+    want = uniform_decode(wl, 400)
+    b, hq, d = wl.q.shape
+    qkv = torch.randn((b, (hq + 16) * d), device=gpu).to(torch.bfloat16)
+    qkv[:, :hq * d] = wl.q.reshape(b, -1)
+    q_view = qkv.split([hq * d, 8 * d, 8 * d], dim=-1)[0].view(b, hq, d)
+    wide = torch.full((b, hq * d + 256), 7.0, dtype=torch.bfloat16, device=gpu)
+    out_view = wide[:, :hq * d].view(b, hq, d)
+    ops.paged_attn_decode(q_view, wl.k_cache, wl.v_cache, wl.block_table, 400, wl.scale, out_view)
+    torch.cuda.synchronize()
+    assert torch.equal(out_view, want) and (wide[:, hq * d:] == 7.0).all()
