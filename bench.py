@@ -31,10 +31,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 # HBM bytes per launch of the decode split kernel on the headline workload.  This is a RECORDED
 # figure, not measured by this run: two `rocprofv3 --pmc` passes of `python3 bench.py --counters`
 # (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch, each scaled by what the same counter reads for the
-# 1 GiB plain copy that run launches first) gave 630,841 KiB read + 4,975 KiB written; the summary is
+# 1 GiB plain copy that run launches first) gave 630,873 KiB read + 4,975 KiB written; the summary is
 # profiles/decode_cfg2_hbm_counters.txt.  The workload is seeded, so the figure only moves when the
 # kernel's access pattern does; it has to be re-recorded then.
-MEASURED_TRAFFIC_BYTES = (630841 + 4975) * 1024
+MEASURED_TRAFFIC_BYTES = (630873 + 4975) * 1024
 TRAFFIC_SOURCE = "recorded: profiles/decode_cfg2_hbm_counters.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)"
 
 
@@ -481,9 +481,15 @@ def main():
                                        cu_seqlens_q=p3.cu_seqlens_q, max_seqlen_k=p3.max_seqlen_k,
                                        cu_seqlens_k=p3.cu_seqlens_k, softmax_scale=p3.scale, causal=True,
                                        block_table=p3.block_table)
+        # the decode op with the batch's length as one host integer (a single kernel, no merge): batch 64 x ctx 2048
+        wu = workloads.make_decode_workload("b64-ctx2048", [2048] * 64, 32, 8, seed=2048, q_scale=128 ** -0.5,
+                                            device=dev, device_fill=True)
+        for _ in range(5):
+            ops.paged_attn_decode(wu.q, wu.k_cache, wu.v_cache, wu.block_table, 2048, wu.scale, out, ws)
         torch.cuda.synchronize()
         pairs = sum((n - c) * c + (n - c) * (n - c + 1) // 2 for n, c in zip(p3.lengths, p3.cached))
         print(json.dumps({"counters_run": True, "copy_bytes": 1 << 30, "decode_algorithmic_bytes": wl.decode_bytes,
+                          "uniform_decode_algorithmic_bytes": wu.decode_bytes,
                           "append_algorithmic_bytes": p3.append_bytes,
                           "fused_algorithmic_bytes": n_q * (2 * hq * d * 2 + 4 * hkv * d * 2),
                           "prefill_flops": 4 * p3.num_q_heads * p3.head_dim * pairs}))
