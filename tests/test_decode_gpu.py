@@ -443,3 +443,22 @@ def test_uniform_form_on_strided_views_and_other_block_sizes(gpu):
     ops.paged_attn_decode(q_view, wl.k_cache, wl.v_cache, wl.block_table, 400, wl.scale, out_view)
     torch.cuda.synchronize()
     assert torch.equal(out_view, want) and (wide[:, hq * d:] == 7.0).all()
+
+
+def test_uniform_form_with_pieces_longer_than_64_blocks(gpu):
+    """Block size 32 and 16,896 tokens: each of the 8 pieces of a sequence spans 66 blocks, two more than
+    the block-id register holds, so the last ones are looked up in the table.  Checked against the tensor
+    form (whose own long-span case is checked against the oracle above)."""
+    length = 8 * 66 * 32
+    wl = workloads.make_decode_workload("uniform-long", [length] * 256, 4, 1, bs=32, seed=9, pool_factor=1.0,
+                                        device=gpu, device_fill=True)
+    got = uniform_decode(wl, length)
+    want = gpu_decode(wl, splits=0)
+    assert np.isfinite(f32(got)).all()
+    assert (got.float() - want.float()).abs().max() <= 8e-3
+    # and one sequence of it against the oracle
+    one = workloads.DecodeWorkload(**{**wl.__dict__, "q": wl.q[:1], "block_table": wl.block_table[:1],
+                                      "context_lens": wl.context_lens[:1], "lengths": wl.lengths[:1],
+                                      "k_new": wl.k_new[:1], "v_new": wl.v_new[:1],
+                                      "slot_mapping": wl.slot_mapping[:1]})
+    assert np.abs(f32(got[:1]) - oracle_decode(one)).max() <= ATTN_ATOL
