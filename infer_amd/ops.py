@@ -178,6 +178,7 @@ def paged_attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
 def paged_attn_decode_split(q, k_cache, v_cache, block_table, context_lens, scale, workspace,
                             split_workgroups: int = 0) -> None:
     """Bandwidth-bound phase alone (partials stay in ``workspace``); for profiling."""
+    assert isinstance(context_lens, torch.Tensor), "the split phase takes the lengths as a tensor"
     b, hq, d, nblk, bs, hkv = _decode_args(q, k_cache, v_cache, context_lens, block_table)
     rc = _lib.load().infer_paged_decode_split_bf16(
         q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), k_cache.stride(0), k_cache.stride(1),
