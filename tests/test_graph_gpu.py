@@ -81,3 +81,40 @@ def test_decode_step_graph_replays_match_eager(gpu):
         wl = workloads.DecodeWorkload("g", hq, hkv, d, bs, d ** -0.5, q[:n], k_new[:n], v_new[:n], k_cache, v_cache,
                                       slots[:n], tables[:n], ctx[:n], list(lengths))
         assert np.abs(f32(got[:n]) - oracle_decode(wl)).max() <= ATTN_ATOL
+
+
+def test_uniform_length_decode_graph_replays_match_eager(gpu):
+    """The single-kernel form (one host integer as the length of every sequence) recorded into a graph:
+    the length is frozen at capture, the tensors it reads are not.  Each replay runs between eager work and
+    synchronisations and is compared with the eager result of the same inputs and with the oracle."""
+    length = 700
+    wl = workloads.make_decode_workload("uniform-graph", [length] * 64, 32, 8, seed=41).to(gpu)
+    out = torch.zeros_like(wl.q)
+    ws = ops.decode_workspace(gpu, 64, 32, 8, 128)
+
+    def step():
+        ops.paged_attn_decode(wl.q, wl.k_cache, wl.v_cache, wl.block_table, length, wl.scale, out, ws)
+
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        step()                                            # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(s)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    g = torch.Generator().manual_seed(42)
+    for replay in range(4):
+        wl.q.copy_(torch.randn(wl.q.shape, generator=g).to(torch.bfloat16))
+        if replay == 2:                                   # another permutation of the same blocks
+            perm = torch.randperm(64, generator=g).to(gpu)
+            wl.block_table.copy_(wl.block_table[perm])
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        out.zero_()
+        step()
+        torch.cuda.synchronize()
+        assert torch.equal(got, out), f"replay {replay} differs from eager"
+        assert np.abs(f32(got) - oracle_decode(wl)).max() <= ATTN_ATOL
