@@ -97,3 +97,23 @@ def test_append_random_case(gpu, seed):
     ops.store_kvcache(key, val, kg, vg, torch.from_numpy(slots.astype(np.int32)).to(gpu))
     torch.cuda.synchronize()
     assert np.array_equal(bits(kg), ek) and np.array_equal(bits(vg), ev), (seed, hkv, d, n, wide)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_decode_uniform_length_random_case(gpu, seed):
+    """The length as one host integer: shapes drawn on both sides of the rule that picks the single-kernel
+    form (batch x KV heads x pieces / 8 workgroups against the compute units), odd lengths, every block size."""
+    rng = np.random.default_rng(3000 + seed)
+    hq, hkv = HEADS[rng.integers(len(HEADS))]
+    bs = int(rng.choice([32, 64, 128, 256]))
+    batch = int(rng.choice([1, 5, 31, 32, 60, 64, 100, 128, 250, 256, 300]))
+    length = int(rng.integers(1, 3000))
+    while batch * length * hq > 2_500_000:     # keeps the CPU oracle to a fraction of a second
+        length = max(1, length // 2)
+    wl = workloads.make_decode_workload(f"uni{seed}", [length] * batch, hq, hkv, bs=bs, seed=seed).to(gpu)
+    out = torch.full_like(wl.q, 3.0)
+    ops.paged_attn_decode(wl.q, wl.k_cache, wl.v_cache, wl.block_table, length, wl.scale, out)
+    torch.cuda.synchronize()
+    got = f32(out)
+    err = float(np.abs(got - oracle_decode(wl)).max())
+    assert np.isfinite(got).all() and err <= ATTN_ATOL, (seed, hq, hkv, bs, batch, length, err)
