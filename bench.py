@@ -95,6 +95,18 @@ def _median_time(fn, min_seconds, min_runs=3, max_runs=50):
     return times[len(times) // 2], len(times)
 
 
+def _cpu_model():
+    """The host CPU's model string (first `model name` of /proc/cpuinfo), for the baseline's record."""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for ln in f:
+                if ln.lower().startswith("model name"):
+                    return ln.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(sample_seqs=16, min_seconds=8.0):
     """The CPU restatement of the same path (gather + SDPA, oracle/torch_path.py) on the host cores,
     over a bounded sample of the same workload: the first ``sample_seqs`` sequences of the batch."""
@@ -110,6 +122,7 @@ def cpu_baseline(sample_seqs=16, min_seconds=8.0):
         "sample": f"first {sample_seqs} of the 64 sequences ({sum(lengths)} tokens, "
                   f"{wl.decode_bytes / 1e6:.1f} MB algorithmic), median of {runs} runs, "
                   f"torch {torch.get_num_threads()} threads",
+        "cpu_model": _cpu_model(),
     }
 
 
