@@ -661,7 +661,8 @@ def main():
     }
     line["prefill_attention"] = {"workload": "cfg3: 16 prompts U[64,2048], 0-50 % cached, causal over the paged cache",
                                  "query_tokens": int(p3.q.shape[0]), "ms": round(pf_ms, 4),
-                                 "TFLOPs": round(pf_flops / (pf_ms * 1e-3) / 1e12, 1)}
+                                 "TFLOPs": round(pf_flops / (pf_ms * 1e-3) / 1e12, 1),
+                                 "frac_of_bf16_mfma_peak": round(pf_flops / (pf_ms * 1e-3) / 1e12 / 2500.0, 4)}
     line["fused_qk_norm_rope_append"] = {"decode_rows": b, "decode_us": fused_small[0],
                                          "prefill_rows": int(p3.q.shape[0]), "prefill_us": fused_big[0],
                                          "prefill_GBps": fused_big[1],
