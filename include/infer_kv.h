@@ -181,7 +181,9 @@ int infer_paged_decode_merge_bf16(void* out, int64_t out_stride0,
  * 80 - 100 % of the compute units for a p in {1, 2, 4, 8}), one kernel streams each sequence in p
  * pieces per KV head, folds them in LDS and writes the result, with no partial results in memory and
  * no merge launch; other shapes run the two kernels of infer_paged_decode_bf16 without reading a
- * lengths array.  The workspace is the one of infer_paged_decode_bf16 (used by the second case). */
+ * lengths array.  The workspace is the one of infer_paged_decode_bf16 (used by the second case).
+ * As for the other decode entries, the first call on a device sets the kernel's LDS limit
+ * (hipFuncSetAttribute): make that call outside stream capture. */
 int infer_paged_decode_uniform_bf16(const void* q, int64_t q_stride0,
                                     const void* k_cache, const void* v_cache,
                                     int64_t cache_block_stride, int64_t cache_token_stride,
