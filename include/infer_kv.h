@@ -37,6 +37,8 @@ extern "C" {
 #define INFER_KV_ESTATE       -5   /* block pool: the call violates an invariant the reference
                                       asserts (double allocate, out of blocks, ...); see
                                       infer_pool_last_error()                                   */
+#define INFER_KV_ENOTINIT     -6   /* first decode call on this device made while its stream is
+                                      being captured: call infer_kv_init() before the capture    */
 
 /* Library version, "major.minor". */
 const char* infer_kv_version(void);
@@ -44,6 +46,13 @@ const char* infer_kv_version(void);
 /* Human-readable text for a code returned by any entry point (negative codes: this library;
  * positive: hipGetErrorString). */
 const char* infer_kv_strerror(int code);
+
+/* One-time set-up for the CURRENT device (host only, no stream work): the decode kernels' LDS limit
+ * (hipFuncSetAttribute), the compute-unit count and the address of the library's own scratch array
+ * (hipGetSymbolAddress).  Every decode entry point does the same on its first call on a device, but
+ * not while its stream is being captured (INFER_KV_ENOTINIT then): a caller that captures HIP graphs
+ * calls this once per device beforehand.  Thread safe; later calls return at once. */
+int infer_kv_init(void);
 
 /* ------------------------------------------------------------------ 1. KV append
  * Replaces store_kvcache / store_kvcache_kernel (infer/ops/attention.py:16-45), called from
@@ -120,19 +129,20 @@ int infer_kv_qk_norm_rope_append_bf16(void* q, int64_t q_stride0, void* k, int64
  * cache_block_stride and token stride cache_token_stride (heads contiguous, D innermost);
  * block_table [B, table_cols] with row stride bt_stride0 >= table_cols; context_lens [B].
  *
- * The work is split across workgroups in equal shares of KV tokens regardless of sequence
- * boundaries; partial (max, sum, accumulator) results go to `workspace` and are merged by a
- * second small kernel.  Size the workspace with infer_paged_decode_workspace_bytes() for the
- * largest batch that will be passed; its contents need no initialisation.  Calls that share a
- * workspace must be ordered on one stream (the records of one call are live until its merge kernel
- * has run); calls on different streams need a workspace each.
+ * The work is cut into equal shares of KV tokens regardless of sequence boundaries, one share per
+ * wavefront.  Partial (max, sum, accumulator) results of one sequence that meet inside a workgroup are
+ * folded there and go to `workspace` as one record; a second small kernel folds the records of a
+ * sequence that reaches into neighbouring workgroups and writes the result.  Size the workspace with
+ * infer_paged_decode_workspace_bytes() for the largest batch that will be passed; its contents need
+ * no initialisation.  Calls that share a workspace must be ordered on one stream (the records of one
+ * call are live until its merge kernel has run); calls on different streams need a workspace each.
  *
- * split_workgroups: workgroups along the KV-split axis of this call, 0 = choose from the device's
- * compute-unit count (the tuned default), at most 1024.  The library keeps no state between calls:
- * two calls may use different counts, also concurrently.
+ * split_workgroups: span positions (workgroups per group of KV heads along the token axis) of this
+ * call, 0 = choose from the device's compute-unit count (the tuned default), at most 1024.  The
+ * library keeps no state between calls: two calls may use different counts, also concurrently.
  *
  * Built for head_dim == 128, 1 <= G <= 16, block_size % 32 == 0 (the reference requires a
- * multiple of 256: infer/config.py:21), num_kv_heads <= 8 or a multiple of 8.
+ * multiple of 256: infer/config.py:21).
  */
 size_t infer_paged_decode_workspace_bytes(int64_t max_batch, int64_t num_q_heads,
                                           int64_t num_kv_heads, int64_t head_dim);
@@ -151,9 +161,10 @@ int infer_paged_decode_bf16(const void* q, int64_t q_stride0,
 
 /* The two phases of infer_paged_decode_bf16 on their own: `split` streams the KV cache and leaves
  * partial results in the workspace, `merge` combines them into `out`.  Calling split then merge
- * on one stream is exactly infer_paged_decode_bf16.  They exist so a profiler or a benchmark can
- * time the bandwidth-bound phase alone.  The merge finds the records from the workspace alone, so
- * it does not need to know the split count. */
+ * on one stream is exactly infer_paged_decode_bf16.  They serve callers that want the partial results
+ * themselves (a context-parallel split across devices would exchange exactly these records) and
+ * profilers that time the bandwidth-bound phase alone.  The merge finds the records from the
+ * workspace alone, so it does not need to know the split count. */
 int infer_paged_decode_split_bf16(const void* q, int64_t q_stride0,
                                   const void* k_cache, const void* v_cache,
                                   int64_t cache_block_stride, int64_t cache_token_stride,
@@ -174,16 +185,13 @@ int infer_paged_decode_merge_bf16(void* out, int64_t out_stride0,
 
 /* The decode call with the context length given as ONE host integer for the whole batch, the
  * `cache_seqlens: int` form of flash_attn_with_kvcache (the function called at
- * infer/ops/attention.py:118-120; the reference itself passes the per-sequence tensor).  Same result
- * as infer_paged_decode_bf16 with context_lens[b] == context_len for every b; context_len == 0
- * gives zeros.  Knowing the length on the host, the library needs no span plan: when batch x KV
- * heads fills the chip with whole workgroups per sequence (batch x num_kv_heads x p / 8 within
- * 80 - 100 % of the compute units for a p in {1, 2, 4, 8}), one kernel streams each sequence in p
- * pieces per KV head, folds them in LDS and writes the result, with no partial results in memory and
- * no merge launch; other shapes run the two kernels of infer_paged_decode_bf16 without reading a
- * lengths array.  The workspace is the one of infer_paged_decode_bf16 (used by the second case).
- * As for the other decode entries, the first call on a device sets the kernel's LDS limit
- * (hipFuncSetAttribute): make that call outside stream capture. */
+ * infer/ops/attention.py:118-120; the reference itself passes the per-sequence tensor, so this form is
+ * NOT on the reference's call path).  Same result as infer_paged_decode_bf16 with
+ * context_lens[b] == context_len for every b; context_len == 0 gives zeros.  Knowing the length, the
+ * host can tell whether every sequence lies inside the spans of one workgroup (batch 64 x 512 ... 4096
+ * tokens on 256 compute units do): the workgroups then write the result themselves and there is no
+ * merge launch; other shapes run the two kernels of infer_paged_decode_bf16 without reading a lengths
+ * array.  The workspace is the one of infer_paged_decode_bf16 (used by the second case). */
 int infer_paged_decode_uniform_bf16(const void* q, int64_t q_stride0,
                                     const void* k_cache, const void* v_cache,
                                     int64_t cache_block_stride, int64_t cache_token_stride,
@@ -199,16 +207,16 @@ int infer_paged_decode_uniform_bf16(const void* q, int64_t q_stride0,
 /* infer_paged_decode_bf16 for callers that cannot allocate and have no workspace to bring: code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in
  * the reference.  Same arguments, result and kernels as infer_paged_decode_bf16 with
- * split_workgroups = 0, but the split-KV partial results go to a fixed array in the library's device
- * image (16 MiB per GPU the library runs on, held until the process ends) instead of a workspace.
- * The call allocates nothing and frees nothing.  Shapes whose partial results do not fit return
- * INFER_KV_EWORKSPACE: the need is about Hkv * (CUs * 8 / Hkv + batch) * 520 * G bytes, i.e. 5.3 MB at
- * batch 64, Hq/Hkv = 32/8 and 8.8 MB at batch 8, 64/8 on 256 compute units, against the
- * INFER_KV_DECODE_NOALLOC_SCRATCH_BYTES of the array.  The array keeps the last
- * call's contents and needs no clearing (every record that is read was written by the same call).
- * All calls on one GPU share it: calls that overlap on one GPU (two streams, two threads) race;
- * calls ordered on one stream are safe.  The first call on a device resolves the array's address
- * (hipGetSymbolAddress); make that call outside stream capture. */
+ * split_workgroups = 0, but the split-KV records go to a fixed array in the library's device image
+ * (16 MiB per GPU the library runs on, held by every process that loads the library until it ends,
+ * whether or not this entry is called) instead of a workspace.  The call allocates nothing and frees
+ * nothing.  Shapes whose records do not fit return INFER_KV_EWORKSPACE: the need is about
+ * Hkv * (CUs * 4 / Hkv + batch) * 520 * G bytes, i.e. 3.2 MB at batch 64, Hq/Hkv = 32/8 and 4.5 MB at
+ * batch 8, 64/8 on 256 compute units, against the INFER_KV_DECODE_NOALLOC_SCRATCH_BYTES of the array.
+ * The array keeps the last call's contents and needs no clearing (every record that is read was
+ * written by the same call).  All calls on one GPU share it: calls that overlap on one GPU (two
+ * streams, two threads) race; calls ordered on one stream are safe.  The address of the array is
+ * resolved by infer_kv_init() or by the first decode call on the device outside stream capture. */
 #define INFER_KV_DECODE_NOALLOC_SCRATCH_BYTES ((size_t)16 << 20)
 int infer_paged_decode_noalloc_bf16(const void* q, int64_t q_stride0,
                                     const void* k_cache, const void* v_cache,

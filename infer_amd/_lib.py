@@ -27,6 +27,7 @@ SIGNATURES = {
     "infer_kv_gather_bf16": (_c.c_int, [_vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp]),
     "infer_kv_qk_norm_rope_append_bf16": (_c.c_int, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _f32, _vp, _i64,
                                                      _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _c.c_int, _vp]),
+    "infer_kv_init": (_c.c_int, []),
     "infer_paged_decode_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64]),
     "infer_paged_decode_bf16": (_c.c_int, [_vp, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _vp,
                                            _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _vp, _sz, _vp]),

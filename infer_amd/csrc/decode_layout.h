@@ -11,7 +11,7 @@
 #define INFER_KV_MAX_SPLIT_WG 1024
 
 struct DecodeWorkspace {
-    size_t header_off;      // int32[64]: {spans used by the last launch, total steps} (diagnostic)
+    size_t header_off;      // int32[64]: {spans used by the last launch, total steps, spans per workgroup and KV head} (diagnostic)
     size_t seg_first_off;   // int32[batch]: first split workgroup that touched the sequence
     size_t seg_last_off;    // int32[batch]: last one
     size_t rec_off;         // [slots] records of rec_stride bytes, one per (segment, KV head)
@@ -29,9 +29,9 @@ static inline size_t align_up_256(size_t x) { return (x + 255) & ~(size_t)255; }
 // padded to a multiple of 16 bytes.
 static inline size_t decode_record_bytes(int64_t group) { return ((size_t)group * 520 + 15) & ~(size_t)15; }
 
-// slots = num_kv_heads * (split_cap + batch): segment (workgroup w < split_cap, sequence b) of KV
-// head h uses slot h * (split_cap + batch) + w + b, which is unique because consecutive segments
-// along the flattened token axis advance w or b (or both) by one.  split_cap is
+// slots = num_kv_heads * (split_cap + batch): the chain of (workgroup span position s < split_cap,
+// sequence b) of KV head h uses slot h * (split_cap + batch) + s + b, which is unique because
+// consecutive chains along the flattened token axis advance s or b (or both) by one.  split_cap is
 // INFER_KV_MAX_SPLIT_WG for a caller-provided workspace; the entry point that brings its own
 // fixed-size scratch lays it out for the split count it launches.
 static inline DecodeWorkspace decode_workspace_layout(int64_t batch, int64_t group, int64_t num_kv_heads,

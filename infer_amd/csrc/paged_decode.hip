@@ -8,13 +8,17 @@
 //
 // Work decomposition
 //   A "step" is 32 consecutive tokens of one sequence (never straddles a cache block because
-//   block_size % 32 == 0).  All steps of all sequences are laid end to end and cut into at
-//   most gridDim.x spans of equal length (to within one step); workgroup x streams span x for up to 8 KV heads, one wavefront per
-//   KV head, so a workgroup reads whole 2 KiB token rows while each wavefront runs its own
-//   private pipeline (no workgroup barrier anywhere).  A span may cover the tail of one
-//   sequence and the head of the next: each (sequence, span) piece is a "segment" and leaves a
-//   partial result (parked in LDS, stored once the wavefront has issued its last load); the merge
-//   kernel folds the segments of a sequence together.
+//   block_size % 32 == 0).  All steps of all sequences are laid end to end and cut into spans of
+//   equal length (to within one step), one per wavefront.  A workgroup is 8 wavefronts: `parts`
+//   consecutive spans for each of 8 / parts KV heads, every wavefront with a private pipeline (no
+//   workgroup barrier while the cache is streamed).  A span may cover the tail of one sequence and
+//   the head of the next: each (sequence, span) piece is a "segment" and leaves a partial result
+//   parked in LDS.  After ONE barrier the segments of a sequence that lie in the same workgroup are
+//   folded through LDS ("chain") and leave one record in the workspace; the merge kernel folds the
+//   records of a sequence that reaches into neighbouring workgroups and writes the bf16 result.  When
+//   the host knows that every sequence lies inside one workgroup (one length for the whole batch that
+//   fits the span grid) the chains are whole sequences: the workgroups write the result themselves
+//   and there is no second launch.
 //
 // Per step and wavefront (KV head h, G = Hq/Hkv query heads):
 //   S^T[token, head] = K[token, :] . Q^T        2 tiles x 4 v_mfma_f32_16x16x32_bf16
@@ -69,9 +73,12 @@ struct DecodeArgs {
     int32_t* seg_last;
     unsigned char* rec; // [slots] partial-result records (layout: decode_record_bytes)
     int rec_stride;
-    int slots_per_head; // records per KV head in the workspace (layout constant, >= gridDim.x + batch)
-    uint16_t* out;      // uniform kernel only: it writes the result itself
+    int slots_per_head; // records per KV head in the workspace (layout constant, >= wg_spans + batch)
+    uint16_t* out;      // [batch, Hq, D] result (only when the workgroups write it themselves)
     int64_t out_stride0;
+    int parts;          // wavefronts (consecutive spans) per KV head in a workgroup: 1, 2, 4 or 8
+    int head_groups;    // workgroups per span position = num_kv_heads / (8 / parts)
+    int wg_spans;       // span positions of the launch; the grid is wg_spans * head_groups workgroups
 };
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 x) { return __builtin_bit_cast(bf16x8, x); }
@@ -142,11 +149,20 @@ __device__ __forceinline__ void lds_order() { __asm__ volatile("" ::: "memory");
 constexpr int kPlanInts = 8;        // ints per segment record
 constexpr int kMaxSegs = 32;        // segments per batch (a span with more is run in several batches)
 constexpr int kPlanBytes = kMaxSegs * kPlanInts * 4;
-// Partial results of finished segments wait in LDS until the wavefront has issued its last load:
-// a global store in the middle of the stream would make the outstanding-load counter unordered
-// (loads and stores share it) and force a full drain of the prefetch pipeline.
-constexpr int kDeferBytes = 8448;   // 4 segments at group size 4, 2 at 8, 1 at 16
-constexpr int kLdsPerWave = kLdsWave + kPlanBytes + kDeferBytes;
+// Partial results wait in LDS until the wavefront has issued its last load: a global store in the
+// middle of the stream would make the outstanding-load counter unordered (loads and stores share
+// it) and force a full drain of the prefetch pipeline.  The area holds one record (the span's first
+// segment when its sequence began in an earlier span or goes on in a later one) and behind it a few
+// results of sequences that lie wholly inside the span.
+constexpr int kDeferBytes = 8448;
+// Per wavefront: what its span left for the fold after the barrier.
+//   ints 0..3  first segment {sequence, flags}
+//   ints 4..7  last segment (only when it is not also the first), same fields
+//   ints 8..15 sequences of the finished results waiting behind the record
+constexpr int kExitBytes = 64;
+constexpr int kLdsPerWave = kLdsWave + kPlanBytes + kDeferBytes + kExitBytes;
+constexpr int kExitValid = 1, kExitLeft = 2, kExitRight = 4;   // flags: entry in use; sequence has earlier / later steps
+constexpr int kMaxRing = 8;
 
 struct SegRec {      // one record of the plan, all wave-uniform
     int b;           // sequence
@@ -192,6 +208,98 @@ struct StepCursor {
     }
 };
 
+// A partial result as one wavefront holds it: lane (g, n), n < G, has columns 16 t + 4 g .. + 3 of
+// query head n in acc[t] (unnormalised), m = running maximum (log2 domain), l = sum, both per head.
+struct Partial {
+    f32x4 acc[8];
+    float m, l;
+};
+
+// (vlane * 8 + t) * 16 is the place of acc[t] in a record, 512 G + 8 n the place of (m, l): the layout
+// of decode_record_bytes().  The same code parks a record in LDS and stores it to the workspace.
+__device__ __forceinline__ void put_record(unsigned char* dst, const Partial& r, int G, int g, int n) {
+    if (n < G) {
+        const int vlane = g * G + n;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) *reinterpret_cast<f32x4*>(dst + (vlane * 8 + t) * 16) = r.acc[t];
+        if (g == 0) *reinterpret_cast<float2*>(dst + 512 * G + n * 8) = make_float2(r.m, r.l);
+    }
+}
+__device__ __forceinline__ void get_record(const unsigned char* src, Partial& r, int G, int g, int n) {
+    const int nn = n < G ? n : 0;   // lanes without a head read head 0's values and never store
+    const int vlane = g * G + nn;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) r.acc[t] = *reinterpret_cast<const f32x4*>(src + (vlane * 8 + t) * 16);
+    const float2 ml = *reinterpret_cast<const float2*>(src + 512 * G + nn * 8);
+    r.m = ml.x;
+    r.l = ml.y;
+}
+
+// into <- into (+) other: the (max, sum) rule of the reference's softmax reduction (softmax.cu:5-16).
+__device__ __forceinline__ void fold(Partial& into, const Partial& other) {
+    const float mn = fmaxf(into.m, other.m);
+    const float f1 = into.m == mn ? 1.f : __builtin_amdgcn_exp2f(into.m - mn);
+    const float f2 = other.m == mn ? 1.f : __builtin_amdgcn_exp2f(other.m - mn);
+#pragma unroll
+    for (int t = 0; t < 8; ++t) into.acc[t] = into.acc[t] * f1 + other.acc[t] * f2;
+    into.l = into.l * f1 + other.l * f2;
+    into.m = mn;
+}
+
+// out[b, h G + n, 16 t + 4 g .. + 3] = acc[t] / l as bf16: four outputs = one 8-byte value per tile.
+__device__ __forceinline__ u32x2 pack_out(const f32x4& v, float inv) {
+    union { __bf16 hv[4]; u32x2 u; } r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) r.hv[e] = (__bf16)(v[e] * inv);
+    return r.u;
+}
+__device__ __forceinline__ void store_out(const DecodeArgs& a, int b, int h, const Partial& r, int G, int g, int n) {
+    if (n < G) {
+        const float inv = r.l > 0.f ? 1.f / r.l : 0.f;
+        uint16_t* op = a.out + (int64_t)b * a.out_stride0 + (int64_t)(h * G + n) * kD + 4 * g;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) *reinterpret_cast<u32x2*>(op + 16 * t) = pack_out(r.acc[t], inv);
+    }
+}
+
+// What a wavefront carries from one batch of segments to the next and to the fold after the barrier.
+struct WaveTail {
+    int flushed;   // segments finished so far
+    int nring;     // finished results waiting in LDS
+};
+
+// Geometry of one wavefront's place in the launch.
+struct WavePlace {
+    int h;       // KV head
+    int s;       // span position of the workgroup (index of its records in the workspace)
+    int lane;
+};
+
+// Writes out the finished results parked behind the record.  kRecords: they are records for the merge
+// kernel (slot = the workgroup's span position + sequence); otherwise bf16 rows of `out`.
+template <bool kRecords>
+__device__ __forceinline__ void drain_ring(const DecodeArgs& a, unsigned char* lds, const WavePlace& wp, WaveTail& wt) {
+    const int G = a.group, g = wp.lane >> 4, n = wp.lane & 15;
+    const unsigned char* ring = lds + kLdsWave + kPlanBytes + a.rec_stride;
+    const int* exitT = reinterpret_cast<const int*>(lds + kLdsWave + kPlanBytes + kDeferBytes);
+    for (int k = 0; k < wt.nring; ++k) {
+        const int b = __builtin_amdgcn_readfirstlane(exitT[8 + k]);
+        if (kRecords) {
+            // the record leaves as it was parked: all 64 lanes, 16 B each, one contiguous run
+            const unsigned char* src = ring + k * a.rec_stride;
+            unsigned char* dst = a.rec + ((int64_t)wp.h * a.slots_per_head + wp.s + b) * a.rec_stride;
+            for (int off = wp.lane * 16; off < a.rec_stride; off += 1024)
+                *reinterpret_cast<u32x4*>(dst + off) = *reinterpret_cast<const u32x4*>(src + off);
+        } else if (n < G) {
+            const unsigned char* src = ring + k * (G * 256) + (g * G + n) * 64;
+            uint16_t* op = a.out + (int64_t)b * a.out_stride0 + (int64_t)(wp.h * G + n) * kD + 4 * g;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) *reinterpret_cast<u32x2*>(op + 16 * t) = *reinterpret_cast<const u32x2*>(src + 8 * t);
+        }
+    }
+    wt.nring = 0;
+}
+
 // Runs one batch of segments for KV head h.
 //
 // Software pipeline (loads return in issue order, so the waits are exact counts): K fragments are
@@ -199,14 +307,15 @@ struct StepCursor {
 // then K(i+2) and V(i+1) are in flight, across sequence boundaries.  Loads past the end of the
 // batch are redirected to one dummy 16-byte location instead of being skipped, which keeps the
 // number of outstanding loads at every wait independent of control flow.
-template <bool kKeep = false>
+template <bool kRecords>
 __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* lds, const int* plan, int nseg,
-                                          int total_steps, int tblv_loaded, int h, int w, int lane) {
+                                          int total_steps, int tblv_loaded, const WavePlace& wp, WaveTail& wt) {
     // The block ids were gathered by vector loads.  Hand them to the loop as a plain register value:
     // otherwise every later read of this register is treated as "may still be in flight" and gets a
     // wait that also drains the K/V loads issued since, which defeats the pipeline.
     int tblv;
     __asm__ volatile("v_mov_b32 %0, %1" : "=v"(tblv) : "v"(tblv_loaded));
+    const int lane = wp.lane, h = wp.h;
     const int g = lane >> 4;   // lane group: the k-slice of MFMA operands, the row-quad of results
     const int n = lane & 15;   // operand row / result column
     const int G = a.group;
@@ -243,11 +352,11 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
         for (int j = 0; j < 4; ++j) qnext[j] = u32x4{0u, 0u, 0u, 0u};
     }
 
-    f32x4 acc[8];
+    Partial cur;
 #pragma unroll
-    for (int t = 0; t < 8; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float m_run = -INFINITY;
-    float l_run = 0.f;
+    for (int t = 0; t < 8; ++t) cur.acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    cur.m = -INFINITY;
+    cur.l = 0.f;
 
     // Row r of K tile t holds token 8 (r / 4) + 4 t + r % 4 of the step, so that result element
     // (tile t, quad element e) of lane group g is token 8 g + (4 t + e): lane group g ends up with
@@ -289,49 +398,57 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
         for (int i = 0; i < 8; ++i) vreg[i] = load16_stream(vb + (i * q_off + lane_off));
     };
 
-    // Partial results: parked in LDS (lane-private layout, valid lanes only), written out by drain().
     unsigned char* defer = lds + kLdsWave + kPlanBytes;
-    const int slot_bytes = a.rec_stride;            // 4G lanes x 8 x 16 B accumulators + G x 8 B (max, sum), padded
-    const int defer_cap = kDeferBytes / slot_bytes; // >= 1 for G <= 16
-    int ndef = 0, first_def = 0;                    // parked segments are first_def .. first_def + ndef - 1
-    const int vlane = g * G + n;                    // index among the 4G lanes that hold real heads
+    int* exitT = reinterpret_cast<int*>(defer + kDeferBytes);
+    // results of sequences that lie wholly inside the span wait behind the record: as records for the
+    // merge kernel (kRecords) or already as the bf16 rows of `out`
+    const int ring_entry = kRecords ? a.rec_stride : G * 256;
+    const int ring_room = (kDeferBytes - a.rec_stride) / ring_entry;
+    const int ring_cap = ring_room < kMaxRing ? ring_room : kMaxRing;   // 0 at group size 16 (and 8 for records)
 
-    auto drain = [&]() {
-        for (int k = 0; k < ndef; ++k) {
-            const int b = __builtin_amdgcn_readfirstlane(plan[(first_def + k) * kPlanInts]);
-            const int64_t slot = (int64_t)h * a.slots_per_head + w + b;
-            // the record leaves as it was parked: all 64 lanes, 16 B each, one contiguous run
-            const unsigned char* src = defer + k * slot_bytes;
-            unsigned char* dst = a.rec + slot * slot_bytes;
-            for (int off = lane * 16; off < slot_bytes; off += 1024)
-                *reinterpret_cast<u32x4*>(dst + off) = *reinterpret_cast<const u32x4*>(src + off);
-        }
-        first_def += ndef;
-        ndef = 0;
-    };
-
-    // Parks the partial result of the segment just finished and resets the accumulators.
+    // The segment just finished leaves its partial result; the accumulators start over.
     auto flush = [&]() {
-        float l_tot = l_run + __shfl_xor(l_run, 16);
+        float l_tot = cur.l + __shfl_xor(cur.l, 16);
         l_tot += __shfl_xor(l_tot, 32);
-        if (ndef == defer_cap) {          // only when one span covers many short sequences
-            lds_order();
-            drain();
-            __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): leave no store in flight behind
-        }
-        unsigned char* dst = defer + ndef * slot_bytes;
+        cur.l = l_tot;
+        const bool left = cseg.s_lo > 0;
+        const bool right = cseg.s_hi < steps_of(cseg.len);
+        const int flags = kExitValid | (left ? kExitLeft : 0) | (right ? kExitRight : 0);
         lds_order();
-        if (n < G) {
+        if (wt.flushed == 0 && (left || right)) {
+            put_record(defer, cur, G, g, n);
+            if (lane == 0) { exitT[0] = cseg.b; exitT[1] = flags; }
+        } else if (right) {
+            // the span's last segment, and not its first: its steps were the last to use the V tile
+            put_record(lds, cur, G, g, n);
+            if (lane == 0) { exitT[4] = cseg.b; exitT[5] = flags; }
+        } else {
+            if (ring_cap > 0 && wt.nring == ring_cap) {   // only when one span covers many short sequences
+                drain_ring<kRecords>(a, lds, wp, wt);
+                __builtin_amdgcn_s_waitcnt(0x0F70);        // vmcnt(0): leave no store in flight behind
+            }
+            if (ring_cap == 0) {
+                if (kRecords) put_record(a.rec + ((int64_t)h * a.slots_per_head + wp.s + cseg.b) * a.rec_stride, cur, G, g, n);
+                else store_out(a, cseg.b, h, cur, G, g, n);
+                __builtin_amdgcn_s_waitcnt(0x0F70);
+            } else {
+                unsigned char* dst = defer + a.rec_stride + wt.nring * ring_entry;
+                if (kRecords) put_record(dst, cur, G, g, n);
+                else if (n < G) {
+                    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
 #pragma unroll
-            for (int t = 0; t < 8; ++t) *reinterpret_cast<f32x4*>(dst + (vlane * 8 + t) * 16) = acc[t];
-            if (g == 0) *reinterpret_cast<float2*>(dst + 512 * G + n * 8) = make_float2(m_run, l_tot);
+                    for (int t = 0; t < 8; ++t) *reinterpret_cast<u32x2*>(dst + (g * G + n) * 64 + 8 * t) = pack_out(cur.acc[t], inv);
+                }
+                if (lane == 0) exitT[8 + wt.nring] = cseg.b;
+                ++wt.nring;
+            }
         }
         lds_order();
-        ++ndef;
+        ++wt.flushed;
 #pragma unroll
-        for (int t = 0; t < 8; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-        m_run = -INFINITY;
-        l_run = 0.f;
+        for (int t = 0; t < 8; ++t) cur.acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        cur.m = -INFINITY;
+        cur.l = 0.f;
     };
 
     auto step = [&](auto PC) {
@@ -365,9 +482,9 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
 #pragma unroll
         for (int i = 1; i < 8; ++i) mx = fmaxf(mx, sv[i]);
         mx = max_xor32(max_xor16(mx));
-        const float m_new = fmaxf(m_run, mx);
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        m_run = m_new;
+        const float m_new = fmaxf(cur.m, mx);
+        const float alpha = __builtin_amdgcn_exp2f(cur.m - m_new);
+        cur.m = m_new;
         float psum = 0.f;
         float pv[8];
 #pragma unroll
@@ -375,7 +492,7 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
             pv[i] = __builtin_amdgcn_exp2f(sv[i] - m_new);
             psum += pv[i];
         }
-        l_run = l_run * alpha + psum;
+        cur.l = cur.l * alpha + psum;
         bf16x8 pb;
 #pragma unroll
         for (int i = 0; i < 8; ++i) pb[i] = (__bf16)pv[i];
@@ -395,7 +512,7 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
 
         if (__any(alpha != 1.f)) {
 #pragma unroll
-            for (int t = 0; t < 8; ++t) acc[t] *= alpha;
+            for (int t = 0; t < 8; ++t) cur.acc[t] *= alpha;
         }
         // ---- O^T += V^T P^T : A operand element i of lane (g, n) is V[token 8 g + i][16 t + n].
         // ds_read_b64_tr_b16: in each group of 16 lanes, lane i points at 4 consecutive elements of
@@ -406,7 +523,7 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
             const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src));
             const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src + 4 * kLdsRow));
             const i16x8 vt = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vt), pb, acc[t], 0, 0, 0);
+            cur.acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vt), pb, cur.acc[t], 0, 0, 0);
         }
         lds_order();
 
@@ -437,177 +554,171 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
     }
     if (i < total_steps) step(P0{});
     lds_order();
-    if (!kKeep) drain();   // kKeep: a single segment whose partial result stays parked in LDS for the caller
 }
 
-// Uniform batch: every sequence has the same number of tokens, known on the host.  A workgroup is
-// 8 wavefronts = (8 / parts) KV heads of ONE sequence x `parts` pieces of its steps.  The pieces of a
-// head are folded through LDS and the workgroup writes the bf16 result itself: no span plan (the
-// block ids are the only load in front of the first K row), no partial result in memory, no merge
-// launch.  The price is that a workgroup reads (8 / parts) x 256 B of every token row instead of
-// the whole 2 KiB row.
-__global__ void __launch_bounds__(512) paged_decode_uniform_kernel(DecodeArgs a, int parts) {
+// kRecords = true: the streaming phase; every chain is left as a record for paged_decode_merge_kernel.
+// kRecords = false: the whole op in one launch, for launches in which the host has made sure that no
+// sequence reaches across two workgroups (every chain is a whole sequence).
+//
+// Grid: wg_spans * head_groups workgroups of 8 wavefronts.  Workgroup (s, hg): wavefront
+// (hsub, piece) streams span s * parts + piece for KV head hg * (8 / parts) + hsub.
+template <bool kRecords>
+__global__ void __launch_bounds__(512) paged_decode_kernel(DecodeArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_all[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int heads_per_wg = 8 / parts;
-    const int wg_per_seq = a.num_kv_heads / heads_per_wg;
-    const int b = blockIdx.x / wg_per_seq;
-    const int h = (blockIdx.x % wg_per_seq) * heads_per_wg + wave / parts;   // consecutive wavefronts: the pieces of one head
-    const int part = wave % parts;
+    const int parts = a.parts;
+    const int hsub = wave / parts, piece = wave - hsub * parts;
+    const int s = blockIdx.x / a.head_groups, hg = blockIdx.x - s * a.head_groups;
+    WavePlace wp;
+    wp.h = hg * (8 / parts) + hsub;
+    wp.s = s;
+    wp.lane = lane;
+    const int h = wp.h;
+    const int w = s * parts + piece;        // this wavefront's span
+    const int W = a.wg_spans * parts;       // spans of the launch
     unsigned char* lds = lds_all + wave * kLdsPerWave;
     int* plan = reinterpret_cast<int*>(lds + kLdsWave);
-    unsigned char* defer = lds + kLdsWave + kPlanBytes;
+    int* exitT = reinterpret_cast<int*>(lds + kLdsWave + kPlanBytes + kDeferBytes);
     const int steps_per_blk = a.block_size / kStep;
-    const int G = a.group;
-    const int g = lane >> 4, n = lane & 15;
-    const int len = a.uniform_len < a.max_ctx ? a.uniform_len : a.max_ctx;
-    const int nsteps = steps_of(len), share = (nsteps + parts - 1) / parts;
-    const int s_lo = part * share, s_hi = s_lo + share < nsteps ? s_lo + share : nsteps;
-    if (s_lo < s_hi) {
-        const int blk0 = s_lo / steps_per_blk;
-        const int nblk = (s_hi - 1) / steps_per_blk - blk0 + 1;
-        if (lane == 0) {
-            plan[0] = b; plan[1] = len; plan[2] = s_lo; plan[3] = s_hi; plan[4] = 0;
-            plan[5] = s_lo - blk0 * steps_per_blk; plan[6] = blk0;
-        }
-        int tblv = 0;   // lane i = i-th block of this piece (a piece of more than 64 blocks looks the rest up)
-        if (lane < nblk) tblv = a.bt[(int64_t)b * a.bt_stride0 + blk0 + lane];
-        lds_order();
-        run_batch<true>(a, lds, plan, 1, s_hi - s_lo, tblv, h, 0, lane);
-    } else if (g == 0 && n < G) {
-        // fewer steps than pieces: an empty piece parks an empty (max, sum)
-        *reinterpret_cast<float2*>(defer + 512 * G + n * 8) = make_float2(-INFINITY, 0.f);
-    }
-    __syncthreads();
-    if (part != 0 || n >= G) return;
-    // piece 0 of every head folds the records of its `parts` pieces (the next wavefronts' LDS areas);
-    // lane (g, n) holds head n, columns 16 t + 4 g .. + 3 of accumulator tile t
-    const int vlane = g * G + n;
-    float m = -INFINITY;
-    for (int p = 0; p < parts; ++p)
-        m = fmaxf(m, reinterpret_cast<const float2*>(defer + p * kLdsPerWave + 512 * G + n * 8)->x);
-    float den = 0.f;
-    f32x4 num[8];
-#pragma unroll
-    for (int t = 0; t < 8; ++t) num[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int p = 0; p < parts; ++p) {
-        const unsigned char* r = defer + p * kLdsPerWave;
-        const float2 ml = *reinterpret_cast<const float2*>(r + 512 * G + n * 8);
-        if (ml.y > 0.f) {
-            const float f = __builtin_amdgcn_exp2f(ml.x - m);
-            den += ml.y * f;
-#pragma unroll
-            for (int t = 0; t < 8; ++t) num[t] += *reinterpret_cast<const f32x4*>(r + (vlane * 8 + t) * 16) * f;
-        }
-    }
-    const float inv = den > 0.f ? 1.f / den : 0.f;
-    uint16_t* op = a.out + (int64_t)b * a.out_stride0 + (int64_t)(h * G + n) * kD + 4 * g;
-#pragma unroll
-    for (int t = 0; t < 8; ++t) {
-        union { __bf16 hv[4]; u32x2 u; } r;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) r.hv[e] = (__bf16)(num[t][e] * inv);
-        *reinterpret_cast<u32x2*>(op + 16 * t) = r.u;
-    }
-}
+    const int G = a.group, g = lane >> 4, n = lane & 15;
 
-__global__ void __launch_bounds__(512) paged_decode_split_kernel(DecodeArgs a) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds_all[];
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int waves = blockDim.x >> 6;
-    const int h = __builtin_amdgcn_readfirstlane(blockIdx.y * waves + wave);
-    const int w = blockIdx.x;
-    const int W = gridDim.x;
-    unsigned char* lds = lds_all + wave * kLdsPerWave;
-    int* plan = reinterpret_cast<int*>(lds + kLdsWave);
-    const int steps_per_blk = a.block_size / kStep;
+    if (lane < kExitBytes / 4) exitT[lane] = 0;
 
-    // total number of steps (the first 64 lengths stay in registers for the second pass)
+    // Total number of steps (the first 64 lengths stay in registers for the second pass).  On the way,
+    // rows without tokens (graph padding) get their zeros: row b from wavefront b / grid of workgroup
+    // b % grid (the merge kernel does it when the chains are left as records).
+    auto zero_rows = [&](int c, int len, bool in_batch) {
+        unsigned long long empty = __ballot(in_batch && len <= 0);
+        while (empty) {
+            const int b = c + __builtin_ctzll(empty);
+            empty &= empty - 1;
+            if (b % (int)gridDim.x == (int)blockIdx.x && (b / (int)gridDim.x) % 8 == wave) {
+                uint16_t* op = a.out + (int64_t)b * a.out_stride0;
+                for (int off = lane * 4; off < a.num_kv_heads * G * kD; off += 256)
+                    *reinterpret_cast<u32x2*>(op + off) = u32x2{0u, 0u};
+            }
+        }
+    };
     const int len0 = lane < a.batch ? ctx_len(a, lane) : 0;
+    if (!kRecords) zero_rows(0, len0, lane < a.batch);
     int total = wave_sum(steps_of(len0));
     for (int c = 64; c < a.batch; c += 64) {
         const int i = c + lane;
-        total += wave_sum(i < a.batch ? steps_of(ctx_len(a, i)) : 0);
+        const int len = i < a.batch ? ctx_len(a, i) : 0;
+        if (!kRecords) zero_rows(c, len, i < a.batch);
+        total += wave_sum(steps_of(len));
     }
     total = __builtin_amdgcn_readfirstlane(total);   // wave-uniform: keep the plan in scalar registers
 
-    // Equal shares: the first `rem` workgroups take one step more.  With fewer steps than workgroups
-    // every step gets a workgroup of its own: on tiny problems a longer span would only serialise
-    // memory latency (measured: one sequence of 512 tokens 14.7 -> 6.7 us).
+    // Equal shares: the first `rem` spans take one step more.  With fewer steps than spans every step
+    // gets a wavefront of its own: on tiny problems a longer span would only serialise memory latency.
     //
-    // A launch takes as long as its longest span (a sweep over forced span counts on 4907 steps:
-    // 102-103 us at 20 steps per workgroup, 104-105 at 22, 108 at 23-24, 113 at 26), so the longest
-    // span is made as short as the grid allows, ceil(total / W) steps, and then the fewest workgroups
-    // that reach it are used: the shares are as even as whole steps permit (4907 steps, 256
-    // workgroups: 246 spans of 19 or 20 steps instead of 42 of 20 and 214 of 19); the workgroups beyond
-    // the span count leave at once.
+    // A launch takes as long as its longest span, so the longest span is made as short as the grid
+    // allows, ceil(total / W) steps, and then the fewest spans that reach it are used: the shares are
+    // as even as whole steps permit; the wavefronts beyond the span count have nothing to stream.
     int spans = W;
     if (total > W) {
         const int longest = (total + W - 1) / W;
         spans = (total + longest - 1) / longest;
     }
-    if (w == 0 && h == 0 && lane == 0) {
+    if (blockIdx.x == 0 && wave == 0 && lane == 0) {
         a.header[0] = spans;
         a.header[1] = total;
+        a.header[2] = parts;
     }
-    if (w >= spans) return;
+    if (s * parts >= spans) return;   // the whole workgroup is beyond the span count
     const int q = total / spans, rem = total - q * spans;
     const int lo = w * q + (w < rem ? w : rem);
-    const int hi = lo + q + (w < rem ? 1 : 0);
-    if (lo >= hi) return;
+    const int hi = w < spans ? lo + q + (w < rem ? 1 : 0) : lo;
 
-    int nseg = 0, nord = 0, nsteps = 0, tblv = 0;
-    int running = 0;
-    for (int c = 0; c < a.batch; c += 64) {
-        const int i = c + lane;
-        const int len = c == 0 ? len0 : (i < a.batch ? ctx_len(a, i) : 0);
-        const int cnt = steps_of(len);
-        const int incl = wave_inclusive_scan(cnt, lane);
-        const int start = running + incl - cnt;
-        const int end = start + cnt;
-        unsigned long long hits = __ballot(cnt > 0 && start < hi && end > lo);
-        while (hits) {
-            const int bit = __builtin_ctzll(hits);
-            hits &= hits - 1;
-            const int st = __builtin_amdgcn_readlane(start, bit);
-            const int en = __builtin_amdgcn_readlane(end, bit);
-            const int ln = __builtin_amdgcn_readlane(len, bit);
-            const int s_lo = (st > lo ? st : lo) - st;
-            const int s_hi = (en < hi ? en : hi) - st;
-            const int b = c + bit;
-            if (h == 0 && lane == 0) {
-                if (s_lo == 0) a.seg_first[b] = w;
-                if (s_hi == en - st) a.seg_last[b] = w;
+    WaveTail wt;
+    wt.flushed = 0;
+    wt.nring = 0;
+    if (lo < hi) {
+        int nseg = 0, nord = 0, nsteps = 0, tblv = 0;
+        int running = 0;
+        for (int c = 0; c < a.batch; c += 64) {
+            const int i = c + lane;
+            const int len = c == 0 ? len0 : (i < a.batch ? ctx_len(a, i) : 0);
+            const int cnt = steps_of(len);
+            const int incl = wave_inclusive_scan(cnt, lane);
+            const int start = running + incl - cnt;
+            const int end = start + cnt;
+            unsigned long long hits = __ballot(cnt > 0 && start < hi && end > lo);
+            while (hits) {
+                const int bit = __builtin_ctzll(hits);
+                hits &= hits - 1;
+                const int st = __builtin_amdgcn_readlane(start, bit);
+                const int en = __builtin_amdgcn_readlane(end, bit);
+                const int ln = __builtin_amdgcn_readlane(len, bit);
+                const int s_lo = (st > lo ? st : lo) - st;
+                const int s_hi = (en < hi ? en : hi) - st;
+                const int b = c + bit;
+                if (kRecords && h == 0 && lane == 0) {
+                    if (s_lo == 0) a.seg_first[b] = s;
+                    if (s_hi == en - st) a.seg_last[b] = s;
+                }
+                const int blk0 = s_lo / steps_per_blk;
+                const int nblk = (s_hi - 1) / steps_per_blk - blk0 + 1;
+                if (nseg == kMaxSegs || (nseg > 0 && nord + nblk > 64)) {
+                    lds_order();
+                    run_batch<kRecords>(a, lds, plan, nseg, nsteps, tblv, wp, wt);
+                    lds_order();
+                    nseg = nord = nsteps = 0;
+                    tblv = 0;
+                }
+                if (lane == 0) {
+                    int* p = plan + nseg * kPlanInts;
+                    p[0] = b; p[1] = ln; p[2] = s_lo; p[3] = s_hi; p[4] = nord; p[5] = s_lo - blk0 * steps_per_blk; p[6] = blk0;
+                }
+                {   // gather this segment's block ids into lanes [nord, nord + nblk)
+                    const int k = lane - nord;
+                    if (k >= 0 && k < nblk && lane < 64) tblv = a.bt[(int64_t)b * a.bt_stride0 + blk0 + k];
+                }
+                ++nseg;
+                nord += nblk;
+                nsteps += s_hi - s_lo;
             }
-            const int blk0 = s_lo / steps_per_blk;
-            const int nblk = (s_hi - 1) / steps_per_blk - blk0 + 1;
-            if (nseg == kMaxSegs || (nseg > 0 && nord + nblk > 64)) {
-                lds_order();
-                run_batch(a, lds, plan, nseg, nsteps, tblv, h, w, lane);
-                lds_order();
-                nseg = nord = nsteps = 0;
-                tblv = 0;
-            }
-            if (lane == 0) {
-                int* p = plan + nseg * kPlanInts;
-                p[0] = b; p[1] = ln; p[2] = s_lo; p[3] = s_hi; p[4] = nord; p[5] = s_lo - blk0 * steps_per_blk; p[6] = blk0;
-            }
-            {   // gather this segment's block ids into lanes [nord, nord + nblk)
-                const int k = lane - nord;
-                if (k >= 0 && k < nblk && lane < 64) tblv = a.bt[(int64_t)b * a.bt_stride0 + blk0 + k];
-            }
-            ++nseg;
-            nord += nblk;
-            nsteps += s_hi - s_lo;
+            running += __builtin_amdgcn_readlane(incl, 63);
+            if (running >= hi) break;
         }
-        running += __builtin_amdgcn_readlane(incl, 63);
-        if (running >= hi) break;
-    }
-    if (nseg > 0) {
+        if (nseg > 0) {
+            lds_order();
+            run_batch<kRecords>(a, lds, plan, nseg, nsteps, tblv, wp, wt);
+        }
         lds_order();
-        run_batch(a, lds, plan, nseg, nsteps, tblv, h, w, lane);
+        drain_ring<kRecords>(a, lds, wp, wt);
+    }
+
+    // ---- the fold: segments of one sequence in consecutive spans of this workgroup form a chain,
+    // folded by the wavefront that holds the chain's first segment
+    __syncthreads();
+    for (int e = 0; e < 2; ++e) {
+        const int* et = exitT + 4 * e;
+        const int flags = __builtin_amdgcn_readfirstlane(et[1]);
+        if (!(flags & kExitValid)) continue;
+        const bool left = flags & kExitLeft;
+        bool right = flags & kExitRight;
+        if (left && piece > 0) continue;   // folded into the chain that began in an earlier wavefront
+        const int b = __builtin_amdgcn_readfirstlane(et[0]);
+        Partial acc;
+        get_record(e == 0 ? lds + kLdsWave + kPlanBytes : lds, acc, G, g, n);
+        for (int p2 = piece + 1; right && p2 < parts; ++p2) {
+            const unsigned char* ow = lds_all + (hsub * parts + p2) * kLdsPerWave + kLdsWave + kPlanBytes;
+            const int f2 = __builtin_amdgcn_readfirstlane(reinterpret_cast<const int*>(ow + kDeferBytes)[1]);
+            if (!(f2 & kExitValid)) break;   // cannot happen: the sequence's next step lies in that span
+            Partial nx;
+            get_record(ow, nx, G, g, n);
+            fold(acc, nx);
+            right = f2 & kExitRight;
+        }
+        if (!kRecords && !left && !right) {   // the whole sequence: this workgroup writes the result
+            store_out(a, b, h, acc, G, g, n);
+            continue;
+        }
+        // (without records every chain is a whole sequence: the host checked the span grid)
+        if (kRecords) put_record(a.rec + ((int64_t)h * a.slots_per_head + s + b) * a.rec_stride, acc, G, g, n);
     }
 }
 
@@ -693,52 +804,114 @@ __global__ void __launch_bounds__(256) paged_decode_merge_kernel(MergeArgs a) {
 
 constexpr int kMaxDevices = 64;
 
-int current_device() {
+}  // namespace
+
+// Scratch of infer_paged_decode_noalloc_bf16: the split-KV records of one call.  Every
+// device the library runs on holds its own copy of this array, at its own address, until the process
+// ends.  In host code the array's NAME is only a handle for hipGetSymbolAddress, never a device address.
+constexpr size_t kNoAllocScratchBytes = INFER_KV_DECODE_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char infer_kv_decode_scratch[kNoAllocScratchBytes];
+
+namespace {
+
+// What the library knows about a device: set once by init_device(), read by every decode call.
+struct DeviceState {
+    int cus;          // compute units
+    void* scratch;    // device address of infer_kv_decode_scratch on this device
+};
+DeviceState g_dev[kMaxDevices];
+bool g_dev_known[kMaxDevices] = {false};
+
+// One-time set-up for the current device: the kernels' LDS limit, the compute-unit count and the
+// address of the scratch array.  Two first calls that race do the same work twice and store the same
+// values.  A first call that arrives while `stream` is being captured is refused: the set-up calls
+// are not stream work and must not run inside a capture.
+int init_device(hipStream_t stream, bool have_stream, const DeviceState** out) {
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
-    return dev;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return INFER_KV_EUNSUPPORTED;
+    if (!__atomic_load_n(&g_dev_known[dev], __ATOMIC_ACQUIRE)) {
+        if (have_stream) {
+            hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+            if (hipStreamIsCapturing(stream, &st) != hipSuccess || st != hipStreamCaptureStatusNone) {
+                (void)hipGetLastError();
+                return INFER_KV_ENOTINIT;
+            }
+        }
+        DeviceState d;
+        d.cus = 0;
+        if (hipDeviceGetAttribute(&d.cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || d.cus <= 0) d.cus = 256;
+        e = hipFuncSetAttribute((const void*)paged_decode_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 8 * kLdsPerWave);
+        if (e != hipSuccess) return (int)e;
+        e = hipFuncSetAttribute((const void*)paged_decode_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 8 * kLdsPerWave);
+        if (e != hipSuccess) return (int)e;
+        d.scratch = nullptr;
+        e = hipGetSymbolAddress(&d.scratch, HIP_SYMBOL(infer_kv_decode_scratch));
+        if (e != hipSuccess) return (int)e;
+        if (d.scratch == nullptr) return INFER_KV_EINVAL;
+        g_dev[dev] = d;
+        __atomic_store_n(&g_dev_known[dev], true, __ATOMIC_RELEASE);
+    }
+    if (out) *out = &g_dev[dev];
+    return INFER_KV_OK;
 }
 
-// Compute units of the current device (cached per device; a benign race writes the same value).
-int device_cu_count() {
-    static int cus[kMaxDevices] = {0};
-    const int dev = current_device();
-    if (cus[dev] == 0) {
-        int v = 0;
-        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) return 256;
-        cus[dev] = v;
-    }
-    return cus[dev];
-}
+// Spans per KV head in a workgroup for the streaming phase.  More of them fold more of a sequence in
+// LDS (fewer records for the merge kernel); fewer make the workgroup read longer contiguous pieces
+// of a token row.  Measured on Qwen3-8B shapes (8 KV heads): 2 is 1-2 % ahead of 1 and of 4 from
+// 1,024 to 32,768 tokens per sequence; 8 (one KV head = 256 B of a row per workgroup) streams 3-6 %
+// slower on contexts of 2,048 tokens and more.
+#ifndef INFER_KV_DECODE_PARTS
+#define INFER_KV_DECODE_PARTS 2
+#endif
 
 struct Launch {
-    int waves;      // wavefronts (KV heads) per workgroup
-    int grid_y;
-    int W;          // workgroups along the KV-split axis
+    int parts;        // wavefronts (consecutive spans) per KV head in a workgroup
+    int head_groups;  // workgroups per span position
+    int S;            // span positions
 };
 
-// split_workgroups: 0 = two wavefronts per SIMD over the whole chip, else the caller's count.
-int plan_launch(int64_t hkv, int64_t split_workgroups, Launch* out) {
-    if (hkv <= 0 || split_workgroups < 0) return INFER_KV_EINVAL;
-    int waves;
-    if (hkv <= 8) waves = (int)hkv;
-    else if (hkv % 8 == 0) waves = 8;
-    else return INFER_KV_EUNSUPPORTED;
-    int64_t W = split_workgroups;
-    if (W == 0) {
-        W = device_cu_count() * 8 / hkv;
-        if (W < 1) W = 1;
+// split_workgroups: span positions of the launch; 0 = as many as fill the chip with one workgroup per
+// compute unit.
+int plan_launch(int64_t hkv, int64_t split_workgroups, int cus, int parts, Launch* out) {
+    if (hkv <= 0 || hkv > (1 << 16) || split_workgroups < 0) return INFER_KV_EINVAL;
+    while (hkv % (8 / parts) != 0) parts *= 2;    // 8 / parts heads per workgroup must divide the heads; parts = 8 always does
+    const int64_t head_groups = hkv / (8 / parts);
+    int64_t S = split_workgroups;
+    if (S == 0) {
+        S = cus / head_groups;
+        if (S < 1) S = 1;
     }
-    if (W > INFER_KV_MAX_SPLIT_WG) W = INFER_KV_MAX_SPLIT_WG;
-    out->waves = waves;
-    out->grid_y = (int)(hkv / waves);
-    out->W = (int)W;
+    if (S > INFER_KV_MAX_SPLIT_WG) S = INFER_KV_MAX_SPLIT_WG;
+    out->parts = parts;
+    out->head_groups = (int)head_groups;
+    out->S = (int)S;
     return INFER_KV_OK;
+}
+
+// One length for the whole batch: does every sequence lie inside one workgroup's spans under launch L?
+// The same arithmetic as the kernel's span plan, so the answer is exact.
+bool sequences_fit_workgroups(int64_t batch, int64_t len, const Launch& L) {
+    if (batch > 4096) return false;               // (the check is a loop over the batch)
+    const int64_t n = (len + kStep - 1) / kStep;  // steps per sequence
+    const int64_t total = batch * n, W = (int64_t)L.S * L.parts;
+    if (n == 0) return true;                      // nothing to attend: the kernel writes the zeros
+    int64_t spans = W;
+    if (total > W) {
+        const int64_t longest = (total + W - 1) / W;
+        spans = (total + longest - 1) / longest;
+    }
+    const int64_t q = total / spans, rem = total - q * spans, big = rem * (q + 1);
+    auto wg_of = [&](int64_t x) { return (x < big ? x / (q + 1) : rem + (x - big) / q) / L.parts; };
+    for (int64_t b = 0; b < batch; ++b)
+        if (wg_of(b * n) != wg_of((b + 1) * n - 1)) return false;
+    return true;
 }
 
 int check_shape(int64_t batch, int64_t hq, int64_t hkv, int64_t d, int64_t bs, int64_t nblk, int64_t table_cols) {
     if (batch <= 0 || hq <= 0 || hkv <= 0 || nblk <= 0 || bs <= 0 || table_cols <= 0) return INFER_KV_EINVAL;
-    if (batch > (1 << 20)) return INFER_KV_EINVAL;
+    if (batch > (1 << 20) || hkv > (1 << 16)) return INFER_KV_EINVAL;
     if (d != kD) return INFER_KV_EUNSUPPORTED;
     if (hq % hkv != 0 || hq / hkv > 16) return INFER_KV_EUNSUPPORTED;
     if (bs % kStep != 0) return INFER_KV_EUNSUPPORTED;
@@ -760,8 +933,9 @@ struct DecodeCall {
     int64_t uniform_len = 0;
 };
 
-// Checks every argument of the split phase and fills in the launch shape.
-int check_split(const DecodeCall& c, int64_t split_workgroups, const void* workspace, Launch* L) {
+// Checks every argument of the streaming phase (host only: no device is touched).
+int check_split(const DecodeCall& c, int64_t split_workgroups, const void* workspace) {
+    if (split_workgroups < 0) return INFER_KV_EINVAL;
     if (!c.q || !c.k_cache || !c.v_cache || !c.block_table || !workspace) return INFER_KV_EINVAL;
     int rc = check_shape(c.batch, c.num_q_heads, c.num_kv_heads, c.head_dim, c.block_size, c.num_blocks, c.table_cols);
     if (rc) return rc;
@@ -773,7 +947,7 @@ int check_split(const DecodeCall& c, int64_t split_workgroups, const void* works
     if (c.batch > 1 && c.bt_stride0 < c.table_cols) return INFER_KV_EINVAL;
     // lane offsets inside one step are kept in 32 bits
     if (32 * c.cache_token_stride >= (int64_t)1 << 31) return INFER_KV_EINVAL;
-    return plan_launch(c.num_kv_heads, split_workgroups, L);
+    return INFER_KV_OK;
 }
 
 int check_out(const void* out, int64_t out_stride0, int64_t num_q_heads) {
@@ -783,8 +957,11 @@ int check_out(const void* out, int64_t out_stride0, int64_t num_q_heads) {
     return INFER_KV_OK;
 }
 
-// Enqueues the split kernel; `base` is device memory laid out as `ws` (arguments already checked).
-int launch_split(const DecodeCall& c, const Launch& L, const DecodeWorkspace& ws, void* base_v, hipStream_t stream) {
+// Enqueues the streaming kernel; `base` is device memory laid out as `ws` (arguments already checked).
+// kRecords: every chain stays in the workspace as a record (out is not touched).
+template <bool kRecords>
+int launch_stream(const DecodeCall& c, const Launch& L, const DecodeWorkspace& ws, void* base_v, void* out,
+                  int64_t out_stride0, hipStream_t stream) {
     DecodeArgs a;
     a.q = (const uint16_t*)c.q;
     a.q_stride0 = c.q_stride0;
@@ -796,8 +973,8 @@ int launch_split(const DecodeCall& c, const Launch& L, const DecodeWorkspace& ws
     a.bt_stride0 = c.bt_stride0;
     a.ctx = c.context_lens;
     a.uniform_len = c.uniform_len > 0x7fffffffLL ? 0x7fffffff : (c.uniform_len < 0 ? 0 : (int)c.uniform_len);
-    a.out = nullptr;
-    a.out_stride0 = 0;
+    a.out = (uint16_t*)out;
+    a.out_stride0 = out_stride0;
     const int64_t max_ctx = c.table_cols * c.block_size;
     a.max_ctx = max_ctx > 0x7fffffffLL ? 0x7fffffff : (int)max_ctx;
     a.batch = (int)c.batch;
@@ -813,74 +990,11 @@ int launch_split(const DecodeCall& c, const Launch& L, const DecodeWorkspace& ws
     a.rec = (unsigned char*)base + ws.rec_off;
     a.rec_stride = (int)ws.rec_stride;
     a.slots_per_head = (int)ws.slots_per_head;
-
-    const size_t lds_bytes = (size_t)L.waves * kLdsPerWave;
-    static bool attr_set[kMaxDevices] = {false};   // the attribute is per device
-    const int dev = current_device();
-    if (!attr_set[dev]) {
-        hipError_t e = hipFuncSetAttribute((const void*)paged_decode_split_kernel,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 8 * kLdsPerWave);
-        if (e != hipSuccess) return (int)e;
-        attr_set[dev] = true;
-    }
-    dim3 grid(L.W, L.grid_y, 1), block(64 * L.waves, 1, 1);
-    hipLaunchKernelGGL(paged_decode_split_kernel, grid, block, lds_bytes, stream, a);
-    return (int)hipGetLastError();
-}
-
-// Pieces per KV head for the uniform kernel, or 0 when the span kernel serves the shape better.  The
-// uniform kernel holds one 8-wavefront workgroup per compute unit (its LDS), so it is used when
-// batch x KV heads x pieces / 8 workgroups fill the chip in one round with even pieces.
-int uniform_parts(const DecodeCall& c) {
-    if (c.uniform_len <= 0 || c.num_kv_heads > (1 << 16)) return 0;
-    const int64_t cus = device_cu_count();
-    const int64_t len = c.uniform_len < c.table_cols * c.block_size ? c.uniform_len : c.table_cols * c.block_size;
-    const int64_t steps = (len + kStep - 1) / kStep;
-    for (int parts = 8; parts >= 1; parts >>= 1) {
-        const int heads_per_wg = 8 / parts;
-        if (c.num_kv_heads % heads_per_wg != 0) continue;
-        const int64_t wgs = c.batch * (c.num_kv_heads / heads_per_wg);
-        if (wgs > cus) continue;
-        if (wgs * 5 < cus * 4) return 0;                        // the largest fit leaves a fifth of the chip idle
-        const int64_t share = (steps + parts - 1) / parts;
-        return steps * 20 >= share * parts * 17 ? parts : 0;    // pieces at least 85 % even
-    }
-    return 0;
-}
-
-int launch_uniform(const DecodeCall& c, void* out, int64_t out_stride0, int parts, hipStream_t stream) {
-    DecodeArgs a{};
-    a.q = (const uint16_t*)c.q;
-    a.q_stride0 = c.q_stride0;
-    a.k = (const uint16_t*)c.k_cache;
-    a.v = (const uint16_t*)c.v_cache;
-    a.blk_stride = c.cache_block_stride;
-    a.tok_stride = c.cache_token_stride;
-    a.bt = c.block_table;
-    a.bt_stride0 = c.bt_stride0;
-    a.ctx = nullptr;
-    a.uniform_len = c.uniform_len > 0x7fffffffLL ? 0x7fffffff : (int)c.uniform_len;
-    const int64_t max_ctx = c.table_cols * c.block_size;
-    a.max_ctx = max_ctx > 0x7fffffffLL ? 0x7fffffff : (int)max_ctx;
-    a.batch = (int)c.batch;
-    a.group = (int)(c.num_q_heads / c.num_kv_heads);
-    a.num_kv_heads = (int)c.num_kv_heads;
-    a.block_size = (int)c.block_size;
-    a.num_blocks = (int)c.num_blocks;
-    a.scale_log2 = c.scale * 1.4426950408889634f;
-    a.rec_stride = (int)decode_record_bytes(a.group);   // layout of a parked partial result
-    a.out = (uint16_t*)out;
-    a.out_stride0 = out_stride0;
-    static bool attr_set[kMaxDevices] = {false};   // the attribute is per device
-    const int dev = current_device();
-    if (!attr_set[dev]) {
-        hipError_t e = hipFuncSetAttribute((const void*)paged_decode_uniform_kernel,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 8 * kLdsPerWave);
-        if (e != hipSuccess) return (int)e;
-        attr_set[dev] = true;
-    }
-    const unsigned wgs = (unsigned)(c.batch * (c.num_kv_heads / (8 / parts)));
-    hipLaunchKernelGGL(paged_decode_uniform_kernel, dim3(wgs, 1, 1), dim3(512, 1, 1), 8 * kLdsPerWave, stream, a, parts);
+    a.parts = L.parts;
+    a.head_groups = L.head_groups;
+    a.wg_spans = L.S;
+    dim3 grid((unsigned)(L.S * L.head_groups), 1, 1), block(512, 1, 1);
+    hipLaunchKernelGGL(paged_decode_kernel<kRecords>, grid, block, 8 * kLdsPerWave, stream, a);
     return (int)hipGetLastError();
 }
 
@@ -905,39 +1019,20 @@ int launch_merge(void* out, int64_t out_stride0, const int32_t* context_lens, in
     return (int)hipGetLastError();
 }
 
-}  // namespace
-
-// Scratch of infer_paged_decode_noalloc_bf16: the split-KV partial results of one call.  Every device
-// the library runs on holds its own copy of this array, at its own address, until the process ends.
-// In host code the array's NAME is only a handle for hipGetSymbolAddress, never a device address.
-constexpr size_t kNoAllocScratchBytes = INFER_KV_DECODE_NOALLOC_SCRATCH_BYTES;
-static __device__ __align__(256) unsigned char infer_kv_decode_scratch[kNoAllocScratchBytes];
-
-namespace {
-
-// Device address of the scratch array on the current device, resolved once per device.
-int noalloc_scratch(void** out) {
-    static void* ptrs[kMaxDevices] = {nullptr};
-    static bool known[kMaxDevices] = {false};
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return (int)e;
-    if (dev < 0 || dev >= kMaxDevices) return INFER_KV_EUNSUPPORTED;
-    if (!__atomic_load_n(&known[dev], __ATOMIC_ACQUIRE)) {      // a race between two first calls resolves the same address twice
-        void* p = nullptr;
-        e = hipGetSymbolAddress(&p, HIP_SYMBOL(infer_kv_decode_scratch));
-        if (e != hipSuccess) return (int)e;
-        if (p == nullptr) return INFER_KV_EINVAL;
-        ptrs[dev] = p;
-        __atomic_store_n(&known[dev], true, __ATOMIC_RELEASE);
-    }
-    *out = ptrs[dev];
-    return INFER_KV_OK;
+// The decode op on memory laid out as `ws`: the streaming kernel and the merge kernel behind it.
+int run_decode(const DecodeCall& c, const Launch& L, const DecodeWorkspace& ws, void* base, void* out,
+               int64_t out_stride0, hipStream_t stream) {
+    int rc = launch_stream<true>(c, L, ws, base, nullptr, 0, stream);
+    if (rc) return rc;
+    return launch_merge(out, out_stride0, c.context_lens, c.uniform_len, c.batch, c.num_q_heads, c.num_kv_heads, ws,
+                        base, stream);
 }
 
 }  // namespace
 
 extern "C" {
+
+int infer_kv_init(void) { return init_device(nullptr, false, nullptr); }
 
 size_t infer_paged_decode_workspace_bytes(int64_t max_batch, int64_t num_q_heads, int64_t num_kv_heads,
                                           int64_t head_dim) {
@@ -958,12 +1053,17 @@ int infer_paged_decode_split_bf16(const void* q, int64_t q_stride0, const void* 
                        table_cols, context_lens, batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks,
                        scale};
     if (!context_lens) return INFER_KV_EINVAL;
-    Launch L;
-    int rc = check_split(c, split_workgroups, workspace, &L);
+    int rc = check_split(c, split_workgroups, workspace);
     if (rc) return rc;
     const DecodeWorkspace ws = decode_workspace_layout(batch, num_q_heads / num_kv_heads, num_kv_heads);
     if (ws.total_bytes > workspace_bytes) return INFER_KV_EWORKSPACE;
-    return launch_split(c, L, ws, workspace, (hipStream_t)stream);
+    const DeviceState* dev = nullptr;
+    rc = init_device((hipStream_t)stream, true, &dev);
+    if (rc) return rc;
+    Launch L;
+    rc = plan_launch(num_kv_heads, split_workgroups, dev->cus, INFER_KV_DECODE_PARTS, &L);
+    if (rc) return rc;
+    return launch_stream<true>(c, L, ws, workspace, nullptr, 0, (hipStream_t)stream);
 }
 
 int infer_paged_decode_merge_bf16(void* out, int64_t out_stride0, const int32_t* context_lens, int64_t batch,
@@ -994,17 +1094,19 @@ int infer_paged_decode_bf16(const void* q, int64_t q_stride0, const void* k_cach
                        scale};
     // everything is checked before the first launch is enqueued
     if (!context_lens) return INFER_KV_EINVAL;
-    Launch L;
-    int rc = check_split(c, split_workgroups, workspace, &L);
+    int rc = check_split(c, split_workgroups, workspace);
     if (rc) return rc;
     rc = check_out(out, out_stride0, num_q_heads);
     if (rc) return rc;
     const DecodeWorkspace ws = decode_workspace_layout(batch, num_q_heads / num_kv_heads, num_kv_heads);
     if (ws.total_bytes > workspace_bytes) return INFER_KV_EWORKSPACE;
-    rc = launch_split(c, L, ws, workspace, (hipStream_t)stream);
+    const DeviceState* dev = nullptr;
+    rc = init_device((hipStream_t)stream, true, &dev);
     if (rc) return rc;
-    return launch_merge(out, out_stride0, context_lens, 0, batch, num_q_heads, num_kv_heads, ws, workspace,
-                        (hipStream_t)stream);
+    Launch L;
+    rc = plan_launch(num_kv_heads, split_workgroups, dev->cus, INFER_KV_DECODE_PARTS, &L);
+    if (rc) return rc;
+    return run_decode(c, L, ws, workspace, out, out_stride0, (hipStream_t)stream);
 }
 
 int infer_paged_decode_uniform_bf16(const void* q, int64_t q_stride0, const void* k_cache, const void* v_cache,
@@ -1017,19 +1119,28 @@ int infer_paged_decode_uniform_bf16(const void* q, int64_t q_stride0, const void
                  table_cols, nullptr, batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, scale};
     c.uniform_len = context_len;
     if (context_len < 0 || context_len > 0x7fffffffLL) return INFER_KV_EINVAL;
-    Launch L;
-    int rc = check_split(c, /*split_workgroups=*/0, workspace, &L);
+    int rc = check_split(c, /*split_workgroups=*/0, workspace);
     if (rc) return rc;
     rc = check_out(out, out_stride0, num_q_heads);
     if (rc) return rc;
     const DecodeWorkspace ws = decode_workspace_layout(batch, num_q_heads / num_kv_heads, num_kv_heads);
     if (ws.total_bytes > workspace_bytes) return INFER_KV_EWORKSPACE;
-    if (const int parts = uniform_parts(c)) return launch_uniform(c, out, out_stride0, parts, (hipStream_t)stream);
-    // shapes the uniform kernel does not fill the chip with: equal spans + merge, without a lengths array
-    rc = launch_split(c, L, ws, workspace, (hipStream_t)stream);
+    const DeviceState* dev = nullptr;
+    rc = init_device((hipStream_t)stream, true, &dev);
     if (rc) return rc;
-    return launch_merge(out, out_stride0, nullptr, context_len, batch, num_q_heads, num_kv_heads, ws, workspace,
-                        (hipStream_t)stream);
+    Launch L;
+    // four spans per KV head in a workgroup, else eight: when every sequence then lies inside one
+    // workgroup, the workgroups write the result themselves and no merge launch follows
+    const int64_t len = context_len < table_cols * block_size ? context_len : table_cols * block_size;
+    for (int parts = 4; parts <= 8; parts *= 2) {
+        rc = plan_launch(num_kv_heads, /*split_workgroups=*/0, dev->cus, parts, &L);
+        if (rc) return rc;
+        if (sequences_fit_workgroups(batch, len, L))
+            return launch_stream<false>(c, L, ws, workspace, out, out_stride0, (hipStream_t)stream);
+    }
+    rc = plan_launch(num_kv_heads, /*split_workgroups=*/0, dev->cus, INFER_KV_DECODE_PARTS, &L);
+    if (rc) return rc;
+    return run_decode(c, L, ws, workspace, out, out_stride0, (hipStream_t)stream);
 }
 
 int infer_paged_decode_noalloc_bf16(const void* q, int64_t q_stride0, const void* k_cache, const void* v_cache,
@@ -1042,21 +1153,21 @@ int infer_paged_decode_noalloc_bf16(const void* q, int64_t q_stride0, const void
                        table_cols, context_lens, batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks,
                        scale};
     if (!context_lens) return INFER_KV_EINVAL;
-    void* scratch = nullptr;
-    int rc = noalloc_scratch(&scratch);
-    if (rc) return rc;
-    Launch L;
-    rc = check_split(c, /*split_workgroups=*/0, scratch, &L);
+    int rc = check_split(c, /*split_workgroups=*/0, /*workspace: the library's own=*/(const void*)16);
     if (rc) return rc;
     rc = check_out(out, out_stride0, num_q_heads);
     if (rc) return rc;
-    // laid out for the split count this call launches, not for the largest one a workspace allows
-    const DecodeWorkspace ws = decode_workspace_layout(batch, num_q_heads / num_kv_heads, num_kv_heads, L.W);
-    if (ws.total_bytes > kNoAllocScratchBytes) return INFER_KV_EWORKSPACE;
-    rc = launch_split(c, L, ws, scratch, (hipStream_t)stream);
+    const DeviceState* dev = nullptr;
+    rc = init_device((hipStream_t)stream, true, &dev);
     if (rc) return rc;
-    return launch_merge(out, out_stride0, context_lens, 0, batch, num_q_heads, num_kv_heads, ws, scratch,
-                        (hipStream_t)stream);
+    void* scratch = dev->scratch;
+    Launch L;
+    rc = plan_launch(num_kv_heads, /*split_workgroups=*/0, dev->cus, INFER_KV_DECODE_PARTS, &L);
+    if (rc) return rc;
+    // laid out for the span positions this call launches, not for the largest count a workspace allows
+    const DecodeWorkspace ws = decode_workspace_layout(batch, num_q_heads / num_kv_heads, num_kv_heads, L.S);
+    if (ws.total_bytes > kNoAllocScratchBytes) return INFER_KV_EWORKSPACE;
+    return run_decode(c, L, ws, scratch, out, out_stride0, (hipStream_t)stream);
 }
 
 }  // extern "C"

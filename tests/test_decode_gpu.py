@@ -215,24 +215,27 @@ def test_random_shapes_and_split_counts(gpu, seed):
 
 @pytest.mark.parametrize("w", [256, 100, 7])
 def test_span_count_reported_in_the_workspace_header(gpu, w):
-    """The split kernel leaves (spans used, total steps) in the first two words of the workspace.  With
-    more steps than workgroups it must use the fewest workgroups that keep the longest span at
-    ceil(total / W) steps, so no workgroup does more than the grid forces; otherwise all of them."""
+    """The streaming kernel leaves (spans used, total steps, spans per workgroup and KV head) in the first
+    words of the workspace.  A launch has W = span positions x spans per workgroup wavefront spans.  With
+    more steps than that it must use the fewest spans that keep the longest one at ceil(total / W) steps,
+    so no wavefront does more than the grid forces; otherwise all of them."""
     for lens in ([4000, 77, 1300, 2048, 31, 900] * 4, [40, 33, 1], workloads.cfg2_lengths(64)):
         wl = workloads.make_decode_workload("hdr", lens, 32, 8, seed=5).to(gpu)
         ws = ops.decode_workspace(gpu, len(lens), 32, 8, 128)
         ops.paged_attn_decode_split(wl.q, wl.k_cache, wl.v_cache, wl.block_table, wl.context_lens, wl.scale, ws,
                                     split_workgroups=w)
         torch.cuda.synchronize()
-        spans, total = (int(v) for v in ws[:8].view(torch.int32)[:2].tolist())
+        spans, total, parts = (int(v) for v in ws[:12].view(torch.int32)[:3].tolist())
         assert total == sum((n + 31) // 32 for n in lens)
-        if total <= w:
-            assert spans == w
+        assert parts in (1, 2, 4, 8)
+        W = w * parts
+        if total <= W:
+            assert spans == W
         else:
-            longest = -(-total // w)
+            longest = -(-total // W)
             assert -(-total // spans) == longest                    # the longest span is as short as W allows
-            assert spans == w or -(-total // (spans - 1)) > longest  # and no fewer workgroups would do
-            assert spans <= w
+            assert spans == W or -(-total // (spans - 1)) > longest  # and no fewer spans would do
+            assert spans <= W
 
 
 def test_cfg2_full_size(gpu):
