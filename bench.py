@@ -17,7 +17,6 @@ front end, the prefill attention, the CPU baselines, and the end-to-end run of t
 from __future__ import annotations
 
 import argparse
-import ctypes
 import json
 import os
 import sys
@@ -51,28 +50,6 @@ def gpu_time_ms(fn, iters, warmup):
     stop.record()
     torch.cuda.synchronize()
     return start.elapsed_time(stop) / iters
-
-
-def load_probe_library():
-    """The measurement-only kernels (read / copy ceilings, the two halves of an append) live in a
-    library of their own, beside the product library."""
-    path = os.path.join(ROOT, "infer_amd", "libinfer_kv_probe.so")
-    if not os.path.exists(path):
-        raise ImportError(f"{path} is not built; run `make -C infer_amd/csrc`")
-    lib = ctypes.CDLL(path)
-    vp, sz, i64 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int64
-    for name, args in {
-        "infer_kv_probe_read": [vp, sz, vp, ctypes.c_int, vp],
-        "infer_kv_probe_read_streaming": [vp, sz, vp, ctypes.c_int, vp],
-        "infer_kv_probe_copy": [vp, vp, sz, ctypes.c_int, vp],
-        "infer_kv_probe_copy_rows": [vp, vp, sz, vp],
-        "infer_kv_probe_read_kv_pattern": [vp, vp, sz, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, ctypes.c_int, vp],
-        "infer_kv_probe_append_read_half": [vp, vp, vp, i64, i64, vp, vp],
-        "infer_kv_probe_append_write_half": [vp, vp, vp, i64, i64, vp],
-    }.items():
-        fn = getattr(lib, name)
-        fn.restype, fn.argtypes = ctypes.c_int, args
-    return lib
 
 
 # ------------------------------------------------------------------------------------------ CPU legs
@@ -182,8 +159,33 @@ def run_e2e(args):
     runner = engine.model_runner
     check = {"steps": 0, "tokens_equal": True, "logits_finite": True, "max_logit_diff": 0.0}
     if not args.e2e_eager and args.e2e_check > 0:
-        runner.check_decode_steps = args.e2e_check      # the runner compares eager and graph on these steps
-        runner.decode_check = check
+        # A decode step is idempotent on the cache (the same row goes to the same slot), so the first
+        # steps run twice on the same state, eagerly and then as the graph replay: same greedy tokens,
+        # finite logits.  The time the check adds is kept apart and taken out of the clock below.
+        replay = runner.decode_hidden
+        left = [args.e2e_check]
+
+        def checked_decode_hidden(run_bs):
+            if left[0] <= 0 or run_bs not in runner.graphs:
+                return replay(run_bs)
+            left[0] -= 1
+            n = int((runner.h_seq_lens[:run_bs] > 0).sum())
+            t0 = time.perf_counter()
+            eager = runner.model.compute_logits(runner._decode_forward(run_bs)[:n]).float()
+            torch.cuda.synchronize()
+            check["seconds"] = check.get("seconds", 0.0) + time.perf_counter() - t0
+            hidden = replay(run_bs)
+            torch.cuda.synchronize()             # the replay itself is the step's own time, not the check's
+            t0 = time.perf_counter()
+            graph = runner.model.compute_logits(hidden[:n]).float()
+            check["steps"] += 1
+            check["tokens_equal"] &= bool(torch.equal(eager.argmax(-1), graph.argmax(-1)))
+            check["logits_finite"] &= bool(torch.isfinite(eager).all() and torch.isfinite(graph).all())
+            check["max_logit_diff"] = max(check["max_logit_diff"], float((eager - graph).abs().max()))
+            torch.cuda.synchronize()
+            check["seconds"] += time.perf_counter() - t0
+            return hidden
+        runner.decode_hidden = checked_decode_hidden
     t0 = time.perf_counter()
     outs = engine.generate(prompts, sp)
     torch.cuda.synchronize()
@@ -307,15 +309,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-curve", action="store_true", help="skip the decode curve of the default run")
     ap.add_argument("--splits", type=int, default=0, help="KV-split workgroups per decode call (0 = library default)")
-    ap.add_argument("--ceiling", action="store_true",
-                    help="measure what this GPU sustains for a read-only stream and a copy (plain kernels of the "
-                         "probe library, same timing method) and print it as JSON; no KV-cache kernel runs")
     ap.add_argument("--counters", action="store_true",
                     help="short untimed run for `rocprofv3 --pmc`: a 1 GiB plain copy (x3), the decode op (x5), "
-                         "a prefill-sized append (x3), its read half and its write half (x3 each), the fused "
-                         "norm + RoPE + append (x3) and the prefill attention (x3) of the same step")
-    ap.add_argument("--append-sweep", action="store_true",
-                    help="KV append rate against the number of rows (64 ... 65,536), printed as JSON")
+                         "a prefill-sized append (x3), the fused norm + RoPE + append (x3) and the prefill "
+                         "attention (x3) of the same step")
     ap.add_argument("--decode-curve", action="store_true", help="only the decode curve, printed as JSON")
     ap.add_argument("--e2e", action="store_true",
                     help="end-to-end decode through the engine (random-init Qwen3, HIP-graph decode) instead "
@@ -339,119 +336,8 @@ def main():
     if args.e2e:
         run_e2e(args)
         return
-    from infer_amd import _lib, ops, workloads
+    from infer_amd import ops, workloads
     dev = torch.device("cuda:0")
-    if args.ceiling:
-        lib = load_probe_library()
-        stream = torch.cuda.current_stream().cuda_stream
-        sink = torch.zeros(4, dtype=torch.uint8, device=dev)
-        res = {"ceiling_run": True, "method": "HIP events, 30 launches after 3 warm-ups, buffers rotated (4 x size)"}
-        for label, nbytes in (("54MB", 13184 * 4096), ("640MB", 640 * 10 ** 6 // 4096 * 4096), ("2GiB", 1 << 31)):
-            bufs = [torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(4)]
-            dsts = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(2)]
-            it = [0]
-
-            def rd(wg):
-                def f():
-                    i = it[0] % 4
-                    it[0] += 1
-                    _lib.check(lib.infer_kv_probe_read(bufs[i].data_ptr(), nbytes, sink.data_ptr(), wg, stream), "probe")
-                return f
-
-            def cp(wg):
-                def f():
-                    i = it[0] % 4
-                    it[0] += 1
-                    _lib.check(lib.infer_kv_probe_copy(bufs[i].data_ptr(), dst.data_ptr(), nbytes, wg, stream), "probe")
-                return f
-
-            def rds(wg):
-                def f():
-                    i = it[0] % 4
-                    it[0] += 1
-                    _lib.check(lib.infer_kv_probe_read_streaming(bufs[i].data_ptr(), nbytes, sink.data_ptr(), wg, stream), "probe")
-                return f
-
-            def cprows():
-                i = it[0] % 4
-                it[0] += 1
-                _lib.check(lib.infer_kv_probe_copy_rows(bufs[i].data_ptr(), dsts[i % 2].data_ptr(), nbytes, stream), "probe")
-            ms = gpu_time_ms(cprows, 32, 4)
-            res[f"copy_one_wave_per_4KiB_{label}_GBps_read_plus_write"] = round(2 * nbytes / ms / 1e6, 1)
-            if label == "54MB":    # the size of one prefill step's append; the other probes are for the large sizes
-                del bufs, dsts
-                continue
-            dst = dsts[0]
-            for wg in (256, 512, 1024):
-                ms = gpu_time_ms(rd(wg), 30, 3)
-                res[f"read_{label}_{wg}wg_GBps"] = round(nbytes / ms / 1e6, 1)
-                ms = gpu_time_ms(rds(wg), 30, 3)
-                res[f"read_streaming_hint_{label}_{wg}wg_GBps"] = round(nbytes / ms / 1e6, 1)
-            for wg in (2048, 8192):
-                ms = gpu_time_ms(cp(wg), 30, 3)
-                res[f"copy_{label}_{wg}wg_GBps_read_plus_write"] = round(2 * nbytes / ms / 1e6, 1)
-            del bufs, dst, dsts
-        # the decode kernel's two read streams (K and V, 1 GiB each) by access pattern and streaming hint
-        tokens = 1 << 19
-        kbuf = torch.empty(tokens * 2048, dtype=torch.uint8, device=dev).random_(0, 255)
-        vbuf = torch.empty(tokens * 2048, dtype=torch.uint8, device=dev).random_(0, 255)
-        for whole, kh, vh in ((0, 0, 0), (0, 0, 1), (0, 1, 1), (1, 0, 0), (1, 0, 1), (1, 1, 0), (1, 1, 1)):
-            ms = gpu_time_ms(lambda: _lib.check(lib.infer_kv_probe_read_kv_pattern(
-                kbuf.data_ptr(), vbuf.data_ptr(), tokens, whole, kh, vh, sink.data_ptr(), 256, stream), "probe"), 8, 2)
-            res[f"kv_streams_2GiB_K_{'rows' if whole else 'mfma_pattern'}_{'hint' if kh else 'plain'}_V_rows_"
-                f"{'hint' if vh else 'plain'}_GBps"] = round(2 * tokens * 2048 / ms / 1e6, 1)
-        print(json.dumps(res))
-        return
-    if args.append_sweep:
-        # KV append from 64 rows (one decode step) to 65,536 rows: launch-bound at the small end, at the
-        # copy rate of the part at the large end.  Sources and destinations rotate over > 512 MB.
-        dkv, res = 1024, {"append_sweep": True, "row_bytes": 2048, "method": "HIP events, 100 launches after 10 warm-ups"}
-        pool_rows = 1 << 18
-        caches = [(torch.empty((pool_rows // 256, 256, 8, 128), dtype=torch.bfloat16, device=dev),
-                   torch.empty((pool_rows // 256, 256, 8, 128), dtype=torch.bfloat16, device=dev)) for _ in range(2)]
-        for n in (64, 256, 1024, 2048, 3072, 4096, 8192, 16384, 32768, 65536):
-            reps = max(2, min(16, (600 << 20) // (n * 4 * dkv)))
-            srcs = [(torch.randn((n, 8, 128), dtype=torch.bfloat16, device=dev),
-                     torch.randn((n, 8, 128), dtype=torch.bfloat16, device=dev)) for _ in range(reps)]
-            slots = [torch.randperm(pool_rows, device=dev)[:n].to(torch.int32) for _ in range(reps)]
-            it = [0]
-
-            def step_append():
-                i = it[0]
-                it[0] += 1
-                kc, vc = caches[i % 2]
-                ops.store_kvcache(srcs[i % reps][0], srcs[i % reps][1], kc, vc, slots[i % reps])
-            ms = gpu_time_ms(step_append, 100, 10)
-            nbytes = workloads.append_algorithmic_bytes(n, n, dkv)
-            res[f"rows_{n}"] = {"us": round(ms * 1e3, 2), "GBps": round(nbytes / ms / 1e6, 1),
-                                "frac_of_8TBps": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
-            del srcs, slots
-        # the same kernel on three slot layouts (the sweep above is the fully scattered one)
-        for n in (13824, 65536):
-            reps = max(2, min(16, (600 << 20) // (n * 4 * dkv)))
-            srcs = [(torch.randn((n, 8, 128), dtype=torch.bfloat16, device=dev),
-                     torch.randn((n, 8, 128), dtype=torch.bfloat16, device=dev)) for _ in range(reps)]
-
-            def whole_blocks():
-                blk = torch.randperm(pool_rows // 256, device=dev)[:n // 256]
-                return (blk[:, None] * 256 + torch.arange(256, device=dev)[None, :]).reshape(-1).to(torch.int32)
-            layouts = {"sequential": [torch.arange(n, device=dev, dtype=torch.int32)] * reps,
-                       "whole_blocks_shuffled": [whole_blocks() for _ in range(reps)],
-                       "rows_scattered": [torch.randperm(pool_rows, device=dev)[:n].to(torch.int32) for _ in range(reps)]}
-            for name, slots in layouts.items():
-                it = [0]
-
-                def step_layout():
-                    i = it[0]
-                    it[0] += 1
-                    kc, vc = caches[i % 2]
-                    ops.store_kvcache(srcs[i % reps][0], srcs[i % reps][1], kc, vc, slots[i % reps])
-                ms = gpu_time_ms(step_layout, 100, 10)
-                nbytes = workloads.append_algorithmic_bytes(n, n, dkv)
-                res[f"layout_{name}_{n}"] = {"us": round(ms * 1e3, 2), "GBps": round(nbytes / ms / 1e6, 1)}
-            del srcs, layouts
-        print(json.dumps(res))
-        return
     if args.decode_curve:
         print(json.dumps({"decode_curve": decode_curve(dev)}))
         return
@@ -460,15 +346,11 @@ def main():
     if args.counters:
         wl = workloads.cfg2(device=dev, device_fill=True)
         b, hq, hkv, d = len(wl.lengths), wl.num_q_heads, wl.num_kv_heads, wl.head_dim
-        probe = load_probe_library()
-        stream = torch.cuda.current_stream().cuda_stream
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
         dst = torch.empty_like(src)
         out = torch.empty((b, hq, d), dtype=torch.bfloat16, device=dev)
         ws = ops.decode_workspace(dev, b, hq, hkv, d)
         p3 = p3_cpu.to(dev)
-        sink = torch.zeros(4, dtype=torch.uint8, device=dev)
-        n3, slots3 = int(p3.slot_mapping.numel()), p3.k_cache.shape[0] * 256
         torch.cuda.synchronize()
         for _ in range(3):
             dst.copy_(src)      # plain copy of known size: 1 GiB read, 1 GiB written
@@ -476,13 +358,6 @@ def main():
             ops.paged_attn_decode(wl.q, wl.k_cache, wl.v_cache, wl.block_table, wl.context_lens, wl.scale, out, ws)
         for _ in range(3):
             ops.store_kvcache(p3.k_new, p3.v_new, p3.k_cache, p3.v_cache, p3.slot_mapping)
-        for _ in range(3):
-            _lib.check(probe.infer_kv_probe_append_read_half(p3.k_new.data_ptr(), p3.v_new.data_ptr(),
-                                                             p3.slot_mapping.data_ptr(), n3, slots3, sink.data_ptr(),
-                                                             stream), "probe")
-        for _ in range(3):
-            _lib.check(probe.infer_kv_probe_append_write_half(p3.k_cache.data_ptr(), p3.v_cache.data_ptr(),
-                                                              p3.slot_mapping.data_ptr(), n3, slots3, stream), "probe")
         n_q = int(p3.q.shape[0])
         qkv = torch.randn((n_q, (hq + 2 * hkv) * d), dtype=torch.bfloat16, device=dev)
         q_, k_, v_ = (t.view(n_q, -1, d) for t in qkv.split([hq * d, hkv * d, hkv * d], dim=-1))
@@ -576,32 +451,6 @@ def main():
 
     ap_ms = gpu_time_ms(append_step, max(args.steps, 48), reps)
     append_gbs = p3.append_bytes / (ap_ms * 1e-3) / 1e9
-    # the two halves of that append on their own (probe library): what its reads and its writes cost alone.
-    # The probe library is measurement scaffolding: without it the two figures are left out, nothing else.
-    rd_ms = wr_ms = None
-    try:
-        probe = load_probe_library()
-    except (ImportError, OSError, AttributeError):
-        probe = None
-    if probe is not None:
-        stream = torch.cuda.current_stream().cuda_stream
-        sink = torch.zeros(4, dtype=torch.uint8, device=dev)
-        n3, slots3 = int(p3.slot_mapping.numel()), p3.k_cache.shape[0] * 256
-
-        def read_half():
-            j = jt[0] % reps
-            jt[0] += 1
-            probe.infer_kv_probe_append_read_half(srcs[j][0].data_ptr(), srcs[j][1].data_ptr(),
-                                                  p3.slot_mapping.data_ptr(), n3, slots3, sink.data_ptr(), stream)
-
-        def write_half():
-            j = jt[0] % reps
-            jt[0] += 1
-            probe.infer_kv_probe_append_write_half(dsts[j][0].data_ptr(), dsts[j][1].data_ptr(),
-                                                   p3.slot_mapping.data_ptr(), n3, slots3, stream)
-        rd_ms = gpu_time_ms(read_half, 48, reps)
-        wr_ms = gpu_time_ms(write_half, 48, reps)
-
     # fused QK-norm + RoPE + append (one launch for the four steps in front of attention), over rotated
     # qkv buffers and cache pairs (> 512 MB in total) so that every launch reads and writes HBM
     def fused_case(n_rows):
@@ -648,16 +497,14 @@ def main():
         "pct_of_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "spin_up_s": spin_up_s,
         "wall_ms_per_step": round(wall_ms, 5),
-        "roofline": {"bound": "hbm", "kernel": "paged_decode_split_kernel", "achieved": round(achieved, 1),
+        "roofline": {"bound": "hbm", "kernel": "paged_decode_kernel<true>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE,
                      "avg_kernel_ms": round(split_ms, 5)},
         "append": {"decode_rows": b, "decode_us": round(ap_small_ms * 1e3, 2),
                    "prefill_rows": int(p3.slot_mapping.numel()), "prefill_bytes": p3.append_bytes,
                    "prefill_us": round(ap_ms * 1e3, 2), "prefill_GBps": round(append_gbs, 1),
-                   "prefill_frac_of_peak": round(append_gbs / HBM_PEAK_GBS, 4),
-                   "read_half_alone_us": round(rd_ms * 1e3, 2) if rd_ms else None,
-                   "write_half_alone_us": round(wr_ms * 1e3, 2) if wr_ms else None},
+                   "prefill_frac_of_peak": round(append_gbs / HBM_PEAK_GBS, 4)},
     }
     line["prefill_attention"] = {"workload": "cfg3: 16 prompts U[64,2048], 0-50 % cached, causal over the paged cache",
                                  "query_tokens": int(p3.q.shape[0]), "ms": round(pf_ms, 4),

@@ -21,6 +21,9 @@
 
 #include "infer_kv/block_pool.hpp"
 
+struct ihipStream_t;   // hipStream_t is a pointer to it (hip/hip_runtime_api.h); named here so that host code
+                       // that only manages a pool does not need the HIP headers
+
 namespace infer {
 
 struct KVCachePoolConfig {
@@ -59,9 +62,15 @@ struct KVCachePoolStats {
 template <typename T>
 class KVCachePool {
 public:
-    // Borrows `storage` (device or host memory of storage_elements() elements).  `stream` is kept
-    // for interface compatibility; nothing here launches work.
+    // The reference's constructor (include/kvcache.hpp:35, cudaStream_t there): the pool allocates its
+    // own device storage for config.num_blocks blocks (hipMalloc, freed by the destructor) and throws
+    // std::runtime_error when the device cannot provide it.
+    explicit KVCachePool(const KVCachePoolConfig& config, ihipStream_t* stream = nullptr);
+    // Borrows `storage` (device or host memory of storage_elements() elements): the form an engine
+    // uses that owns the cache as one tensor sized from free memory.  `stream` is kept for interface
+    // compatibility; nothing here launches work.
     KVCachePool(const KVCachePoolConfig& config, T* storage, void* stream = nullptr);
+    ~KVCachePool();
     KVCachePool(const KVCachePool&) = delete;
     KVCachePool& operator=(const KVCachePool&) = delete;
 
@@ -93,6 +102,7 @@ private:
 
     KVCachePoolConfig config_;
     T* storage_;
+    bool owns_storage_ = false;
     void* stream_;
     BlockPool pool_;
     std::unordered_map<size_t, Seq> seqs_;

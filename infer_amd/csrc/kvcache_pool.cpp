@@ -2,6 +2,7 @@
 #include "infer_kv/kvcache.hpp"
 
 #include <hip/hip_bfloat16.h>
+#include <hip/hip_runtime_api.h>
 
 #include <iostream>
 #include <stdexcept>
@@ -15,6 +16,28 @@ KVCachePool<T>::KVCachePool(const KVCachePoolConfig& config, T* storage, void* s
     if (!storage) throw std::invalid_argument("KVCachePool: storage is null");
     if (config.head_size == 0 || config.num_heads == 0 || config.num_layers == 0)
         throw std::invalid_argument("KVCachePool: empty geometry");
+}
+
+template <typename T>
+KVCachePool<T>::KVCachePool(const KVCachePoolConfig& config, ihipStream_t* stream)
+    : config_(config), storage_(nullptr), owns_storage_(true), stream_(stream),
+      pool_(static_cast<int32_t>(config.num_blocks), static_cast<int32_t>(config.block_size)) {
+    if (config.head_size == 0 || config.num_heads == 0 || config.num_layers == 0)
+        throw std::invalid_argument("KVCachePool: empty geometry");
+    void* p = nullptr;
+    const size_t bytes = storage_elements(config) * sizeof(T);
+    const hipError_t e = hipMalloc(&p, bytes);
+    if (e != hipSuccess || p == nullptr) {
+        (void)hipGetLastError();
+        throw std::runtime_error("KVCachePool: cannot allocate " + std::to_string(bytes) + " bytes of device memory: " +
+                                 hipGetErrorString(e));
+    }
+    storage_ = static_cast<T*>(p);
+}
+
+template <typename T>
+KVCachePool<T>::~KVCachePool() {
+    if (owns_storage_ && storage_) (void)hipFree(storage_);
 }
 
 template <typename T>

@@ -114,6 +114,8 @@ def decode_workspace(device, max_batch: int, num_q_heads: int, num_kv_heads: int
     ws = _workspaces.get(key)
     if ws is None or ws[0] < max_batch:
         cap = max(max_batch, 64 if ws is None else 2 * ws[0])
+        with torch.cuda.device(device):      # the library's per-device set-up, before any graph capture
+            _lib.check(_lib.load().infer_kv_init(), "infer_kv_init")
         nbytes = _lib.load().infer_paged_decode_workspace_bytes(cap, num_q_heads, num_kv_heads, head_dim)
         if nbytes == 0:
             raise RuntimeError("paged decode: unsupported shape "

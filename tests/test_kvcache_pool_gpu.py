@@ -18,7 +18,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def test_views_feed_append_and_decode(gpu, tmp_path):
     exe = os.path.join(ROOT, "tests", "cpp", "test_kvcache_pool_gpu")
-    assert os.path.exists(exe), "build it with `make -C infer_amd/csrc`"
+    assert os.path.exists(exe), "build it with `make -C infer_amd/csrc tests`"
     run = subprocess.run([exe, str(tmp_path)], capture_output=True, text=True, timeout=120)
     assert run.returncode == 0 and run.stdout.strip().endswith("ok"), run.stdout + run.stderr
 
