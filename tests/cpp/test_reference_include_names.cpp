@@ -14,28 +14,28 @@
 #include <cstdio>
 #include <stdexcept>
 
-#define CHECK(c) do { if (!(c)) { std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #c); return 1; } } while (0)
+#define REQUIRE(c) do { if (!(c)) { std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #c); return 1; } } while (0)
 
 int main() {
     using T = hip_bfloat16;
     // operator API: nothing registered yet -> nullptr, as in the reference (opregistry.hpp:25-40)
     auto& reg = infer::OperatorRegistry::getInstance();
-    CHECK((reg.getOperator<T, infer::KVAppendOperator>(infer::OperatorType::KV_APPEND, "KV_APPEND") == nullptr));
+    REQUIRE((reg.getOperator<T, infer::KVAppendOperator>(infer::OperatorType::KV_APPEND, "KV_APPEND") == nullptr));
     infer::OperatorFactory::registerOperators<T>();
     auto app = infer::OperatorFactory::getKVAppendOperator<T>();
     auto att = infer::OperatorFactory::getPagedAttentionOperator<T>();
-    CHECK(app && att);
-    CHECK(app->type() == infer::OperatorType::KV_APPEND && app->name() == "KV_APPEND");
-    CHECK(att->type() == infer::OperatorType::PAGED_ATTENTION);
+    REQUIRE(app && att);
+    REQUIRE(app->type() == infer::OperatorType::KV_APPEND && app->name() == "KV_APPEND");
+    REQUIRE(att->type() == infer::OperatorType::PAGED_ATTENTION);
     infer::Operator* base = app.get();       // really an Operator
-    CHECK(base->name() == "KV_APPEND");
+    REQUIRE(base->name() == "KV_APPEND");
     bool threw = false;
     try {
         infer::OperatorFactory::registerOperators<float>();   // the macro instantiates bf16 only
     } catch (const std::runtime_error&) {
         threw = true;
     }
-    CHECK(threw);
+    REQUIRE(threw);
     infer::UnifiedOp<T> unified;
     (void)unified;
 
@@ -47,24 +47,24 @@ int main() {
     const bool have_gpu = hipGetDeviceCount(&devices) == hipSuccess && devices > 0;
     try {
         infer::KVCachePool<T> pool(cfg, stream);
-        CHECK(have_gpu);
+        REQUIRE(have_gpu);
         pool.prefetch_sequence(7, 300);
         auto k = pool.get_key_cache(7, 1);
         auto v = pool.get_value_cache(7, 1);
-        CHECK(k.base != nullptr && v.base != nullptr && k.base != v.base);
-        CHECK(k.num_blocks_used == 2 && k.block_size == 256 && k.num_heads == 8 && k.head_size == 128);
-        CHECK(hipMemset(k.base, 0, 16) == hipSuccess);        // device memory the pool allocated
+        REQUIRE(k.base != nullptr && v.base != nullptr && k.base != v.base);
+        REQUIRE(k.num_blocks_used == 2 && k.block_size == 256 && k.num_heads == 8 && k.head_size == 128);
+        REQUIRE(hipMemset(k.base, 0, 16) == hipSuccess);        // device memory the pool allocated
         threw = false;
         try {
             pool.get_key_cache(8, 0);
         } catch (const std::runtime_error&) {                 // unknown sequence: src/kvcache.cc:38-41
             threw = true;
         }
-        CHECK(threw);
+        REQUIRE(threw);
         pool.free_sequence(7);
-        CHECK(pool.free_blocks() == 8);
+        REQUIRE(pool.free_blocks() == 8);
     } catch (const std::runtime_error& e) {
-        CHECK(!have_gpu);                                     // without a device the allocation must throw, nothing else
+        REQUIRE(!have_gpu);                                     // without a device the allocation must throw, nothing else
         std::printf("no device: %s\n", e.what());
     }
     std::printf("ok\n");

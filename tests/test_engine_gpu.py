@@ -154,6 +154,58 @@ def test_graph_replays_at_qwen3_8b_layer_shapes_match_eager(gpu):
         sched.postprocess(batch, tokens)
 
 
+def test_qwen3_8b_geometry_prefill_and_decode_steps_match_oracle(gpu):
+    """Two layers of the Qwen3-8B geometry of the end-to-end configuration (hidden 4096, 32 query and 8 KV
+    heads of 128, intermediate 12288), batch 16 with mixed prompt lengths on both sides of a block
+    boundary: one prefill and three decode steps, the decode steps as HIP-graph replays.  The logits of
+    every step are compared with the float32 whole-sequence oracle (one oracle pass per sequence over its
+    final tokens gives the rows of all four steps: dense causal attention does not look ahead)."""
+    from infer_amd.layers import cos_sin_table
+    from infer_amd.model_runner import ModelRunner
+    from infer_amd.scheduler import Scheduler
+    from infer_amd.sequence import Sequence
+    hf = ModelConfig(vocab_size=2048, hidden_size=4096, intermediate_size=12288, num_hidden_layers=2,
+                     num_attention_heads=32, num_key_value_heads=8, head_dim=128, max_position_embeddings=4096)
+    config = Config(hf_config=hf, num_kvcache_blocks=64, max_model_len=4096, max_num_batched_tokens=16384,
+                    max_num_seqs=16, enforce_eager=False, seed=5)
+    runner = ModelRunner(config)
+    sched = Scheduler(config)
+    g = np.random.default_rng(2)
+    lengths = [3, 17, 64, 100, 129, 200, 254, 255, 256, 257, 300, 31, 150, 90, 222, 400]
+    seqs = [Sequence([int(t) for t in g.integers(0, hf.vocab_size, size=n)], SamplingParams(0.0, 4, True))
+            for n in lengths]
+    for s in seqs:
+        sched.add(s)
+    rows = {id(s): [] for s in seqs}            # logits of each step, per sequence
+    for step in range(4):
+        batch, is_prefill = sched.schedule()
+        assert is_prefill == (step == 0) and len(batch) == 16
+        if not is_prefill:
+            assert runner.prepare_decode(batch) in runner.graphs     # the step below is a graph replay
+        logits = runner.run_model(batch, is_prefill)
+        reset_context()
+        assert torch.isfinite(logits.float()).all()
+        for s, row in zip(batch, logits.float().cpu()):
+            rows[id(s)].append(row)
+        sched.postprocess(batch, logits.float().argmax(dim=-1).tolist())
+    weights = {k: v.detach().float().cpu() for k, v in runner.model.named_parameters()}
+    table = cos_sin_table(hf.head_dim, hf.max_position_embeddings, hf.rope_theta, runner.device).float().cpu()
+    worst = 0.0
+    for s in seqs:
+        n = s.num_prompt_tokens
+        fed = s.token_ids[:n + 3]               # the prompt and the three tokens fed by the decode steps
+        pos = qwen3_ref.engine_positions(n, len(fed), config.decode_position_offset)
+        want = qwen3_ref.forward_full(weights, hf, fed, pos, table)
+        for k, got in enumerate(rows[id(s)]):
+            ref = want[n - 1 + k]
+            scale = ref.abs().max().item()
+            err = (got - ref).abs().max().item()
+            worst = max(worst, err / scale)
+            assert err <= LOGIT_TOL * scale, (n, k, err, scale)
+            assert ref.max().item() - ref[int(got.argmax())].item() <= 2 * LOGIT_TOL * scale
+    print("8B-geometry logits: worst error relative to the largest logit", worst)
+
+
 def test_generate_graph_and_eager_agree_and_prefix_cache_hits(gpu):
     from infer_amd.llm_engine import LLMEngine
     ps = prompts([30, 130, 260, 511], seed=5)
