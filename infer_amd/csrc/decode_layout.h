@@ -10,11 +10,16 @@
 // where every record lives whatever split count a call asks for.
 #define INFER_KV_MAX_SPLIT_WG 1024
 
+// The first pieces of every sequence have records at fixed places, [batch][KV head][this many], so that
+// the merge kernel can request them before it has read how many pieces a sequence has.
+#define INFER_KV_DECODE_FIRST_PIECES 4
+
 struct DecodeWorkspace {
     size_t header_off;      // int32[64]: {spans used by the last launch, total steps, spans per workgroup and KV head} (diagnostic)
     size_t seg_first_off;   // int32[batch]: first split workgroup that touched the sequence
     size_t seg_last_off;    // int32[batch]: last one
-    size_t rec_off;         // [slots] records of rec_stride bytes, one per (segment, KV head)
+    size_t rec_first_off;   // [batch][KV heads][INFER_KV_DECODE_FIRST_PIECES] records: pieces 0 .. 3 of every sequence
+    size_t rec_off;         // [slots] records of rec_stride bytes: later pieces, one per (span position, sequence, KV head)
     size_t rec_stride;      // bytes per record, a multiple of 16
     int64_t slots_per_head; // records per KV head: split_cap + batch
     size_t total_bytes;
@@ -44,6 +49,7 @@ static inline DecodeWorkspace decode_workspace_layout(int64_t batch, int64_t gro
     ws.seg_first_off = off;   off = align_up_256(off + (size_t)batch * sizeof(int32_t));
     ws.seg_last_off = off;    off = align_up_256(off + (size_t)batch * sizeof(int32_t));
     ws.rec_stride = decode_record_bytes(group);
+    ws.rec_first_off = off;   off = align_up_256(off + (size_t)batch * (size_t)num_kv_heads * INFER_KV_DECODE_FIRST_PIECES * ws.rec_stride);
     ws.rec_off = off;         off = align_up_256(off + slots * ws.rec_stride);
     ws.total_bytes = off;
     return ws;

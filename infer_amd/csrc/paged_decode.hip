@@ -71,7 +71,8 @@ struct DecodeArgs {
     int32_t* header;
     int32_t* seg_first;
     int32_t* seg_last;
-    unsigned char* rec; // [slots] partial-result records (layout: decode_record_bytes)
+    unsigned char* rec; // [slots] partial-result records (layout: decode_record_bytes): pieces kFirstPieces and later of a sequence
+    unsigned char* rec_first; // [batch][KV head][kFirstPieces] records: the first pieces of every sequence, at places the merge kernel knows in advance
     int rec_stride;
     int slots_per_head; // records per KV head in the workspace (layout constant, >= wg_spans + batch)
     uint16_t* out;      // [batch, Hq, D] result (only when the workgroups write it themselves)
@@ -156,13 +157,14 @@ constexpr int kPlanBytes = kMaxSegs * kPlanInts * 4;
 // results of sequences that lie wholly inside the span.
 constexpr int kDeferBytes = 8448;
 // Per wavefront: what its span left for the fold after the barrier.
-//   ints 0..3  first segment {sequence, flags}
+//   ints 0..3  first segment {sequence, flags, position of the sequence's first step on the step axis}
 //   ints 4..7  last segment (only when it is not also the first), same fields
 //   ints 8..15 sequences of the finished results waiting behind the record
 constexpr int kExitBytes = 64;
 constexpr int kLdsPerWave = kLdsWave + kPlanBytes + kDeferBytes + kExitBytes;
 constexpr int kExitValid = 1, kExitLeft = 2, kExitRight = 4;   // flags: entry in use; sequence has earlier / later steps
 constexpr int kMaxRing = 8;
+constexpr int kFirstPieces = INFER_KV_DECODE_FIRST_PIECES;
 
 struct SegRec {      // one record of the plan, all wave-uniform
     int b;           // sequence
@@ -171,6 +173,7 @@ struct SegRec {      // one record of the plan, all wave-uniform
     int ord0;        // block ordinal of the first step's block
     int in0;         // step index of s_lo inside its block
     int blk0;        // index of that block in the sequence's table row
+    int st;          // position of the sequence's first step on the step axis
 };
 
 __device__ __forceinline__ SegRec read_rec(const int* plan, int seg) {
@@ -183,6 +186,7 @@ __device__ __forceinline__ SegRec read_rec(const int* plan, int seg) {
     r.ord0 = __builtin_amdgcn_readfirstlane(p[4]);
     r.in0 = __builtin_amdgcn_readfirstlane(p[5]);
     r.blk0 = __builtin_amdgcn_readfirstlane(p[6]);
+    r.st = __builtin_amdgcn_readfirstlane(p[7]);
     return r;
 }
 
@@ -275,6 +279,16 @@ struct WavePlace {
     int lane;
 };
 
+// Where the record of (sequence b, KV head h) from the workgroup at span position s goes: the sequence's
+// piece number is s minus the span position of its first step; the first kFirstPieces pieces have fixed
+// places (the merge kernel requests them before it knows how many there are), later ones the slot
+// h * slots_per_head + s + b, unique because consecutive chains advance s or b.
+__device__ __forceinline__ unsigned char* record_place(const DecodeArgs& a, int b, int h, int s, int s_first) {
+    const int k = s - s_first;
+    if (k < kFirstPieces) return a.rec_first + (((int64_t)b * a.num_kv_heads + h) * kFirstPieces + k) * a.rec_stride;
+    return a.rec + ((int64_t)h * a.slots_per_head + s + b) * a.rec_stride;
+}
+
 // Writes out the finished results parked behind the record.  kRecords: they are records for the merge
 // kernel (slot = the workgroup's span position + sequence); otherwise bf16 rows of `out`.
 template <bool kRecords>
@@ -287,7 +301,7 @@ __device__ __forceinline__ void drain_ring(const DecodeArgs& a, unsigned char* l
         if (kRecords) {
             // the record leaves as it was parked: all 64 lanes, 16 B each, one contiguous run
             const unsigned char* src = ring + k * a.rec_stride;
-            unsigned char* dst = a.rec + ((int64_t)wp.h * a.slots_per_head + wp.s + b) * a.rec_stride;
+            unsigned char* dst = record_place(a, b, wp.h, 0, 0);   // a whole sequence: its only piece
             for (int off = wp.lane * 16; off < a.rec_stride; off += 1024)
                 *reinterpret_cast<u32x4*>(dst + off) = *reinterpret_cast<const u32x4*>(src + off);
         } else if (n < G) {
@@ -417,18 +431,18 @@ __device__ __forceinline__ void run_batch(const DecodeArgs& a, unsigned char* ld
         lds_order();
         if (wt.flushed == 0 && (left || right)) {
             put_record(defer, cur, G, g, n);
-            if (lane == 0) { exitT[0] = cseg.b; exitT[1] = flags; }
+            if (lane == 0) { exitT[0] = cseg.b; exitT[1] = flags; exitT[2] = cseg.st; }
         } else if (right) {
             // the span's last segment, and not its first: its steps were the last to use the V tile
             put_record(lds, cur, G, g, n);
-            if (lane == 0) { exitT[4] = cseg.b; exitT[5] = flags; }
+            if (lane == 0) { exitT[4] = cseg.b; exitT[5] = flags; exitT[6] = cseg.st; }
         } else {
             if (ring_cap > 0 && wt.nring == ring_cap) {   // only when one span covers many short sequences
                 drain_ring<kRecords>(a, lds, wp, wt);
                 __builtin_amdgcn_s_waitcnt(0x0F70);        // vmcnt(0): leave no store in flight behind
             }
             if (ring_cap == 0) {
-                if (kRecords) put_record(a.rec + ((int64_t)h * a.slots_per_head + wp.s + cseg.b) * a.rec_stride, cur, G, g, n);
+                if (kRecords) put_record(record_place(a, cseg.b, h, 0, 0), cur, G, g, n);
                 else store_out(a, cseg.b, h, cur, G, g, n);
                 __builtin_amdgcn_s_waitcnt(0x0F70);
             } else {
@@ -671,6 +685,7 @@ __global__ void __launch_bounds__(512) paged_decode_kernel(DecodeArgs a) {
                 if (lane == 0) {
                     int* p = plan + nseg * kPlanInts;
                     p[0] = b; p[1] = ln; p[2] = s_lo; p[3] = s_hi; p[4] = nord; p[5] = s_lo - blk0 * steps_per_blk; p[6] = blk0;
+                    p[7] = st;
                 }
                 {   // gather this segment's block ids into lanes [nord, nord + nblk)
                     const int k = lane - nord;
@@ -718,7 +733,13 @@ __global__ void __launch_bounds__(512) paged_decode_kernel(DecodeArgs a) {
             continue;
         }
         // (without records every chain is a whole sequence: the host checked the span grid)
-        if (kRecords) put_record(a.rec + ((int64_t)h * a.slots_per_head + s + b) * a.rec_stride, acc, G, g, n);
+        if (kRecords) {
+            // span position of the workgroup that holds the sequence's first step
+            const int st = __builtin_amdgcn_readfirstlane(et[2]);
+            const int big = rem * (q + 1);
+            const int sp = st < big ? st / (q + 1) : rem + (q > 0 ? (st - big) / q : 0);
+            put_record(record_place(a, b, h, s, sp / parts), acc, G, g, n);
+        }
     }
 }
 
@@ -728,77 +749,104 @@ struct MergeArgs {
     const int32_t* ctx;     // nullptr: every sequence has uniform_len tokens
     int uniform_len;
     int group;
+    int num_kv_heads;
     int slots_per_head;     // records per KV head in the workspace, as in the split launch
     const int32_t* seg_first;
     const int32_t* seg_last;
     const unsigned char* rec;
+    const unsigned char* rec_first;
     int rec_stride;
     int batch;
 };
 
-// grid (batch, Hq), 256 threads = 8 segment lanes x 32 column quads.  Thread (j, c) folds segments
-// j, j + 8, ... of its (sequence, query head) for output columns 4c .. 4c+3 with the running
-// (max, sum) rule; the eight lanes are then folded through LDS.  All loads of a thread are
-// independent, so a sequence cut into many segments costs about one memory round trip.
+// Grid (batch, KV heads), 4 wavefronts: the workgroup folds the records of one sequence for the whole
+// GQA group of a KV head (they are contiguous in a record).  Wavefront j takes pieces j, j + 4, ... of
+// the sequence; lane c the 16-byte vectors c, c + 64, ... of a record (NU of them: 32 G / 64), each
+// with the (max, sum) of its head.  The first kFirstPieces pieces sit at places that depend only on
+// (sequence, KV head, piece), so they are requested together with the sequence's length and piece
+// range, before either is known: one memory round trip for a sequence of up to four pieces.  The four
+// wavefronts are then folded through LDS in piece order.
+template <int NU>
 __global__ void __launch_bounds__(256) paged_decode_merge_kernel(MergeArgs a) {
-    __shared__ float red[8][32][6];
-    const int b = blockIdx.x;
-    const int head = blockIdx.y;
+    static_assert(kFirstPieces == 4, "one wavefront per fixed place");
+    extern __shared__ __attribute__((aligned(16))) unsigned char red[];   // [3 wavefronts][NU][64 lanes] f32x4, then as many float2
+    f32x4* red_num = reinterpret_cast<f32x4*>(red);
+    float2* red_ml = reinterpret_cast<float2*>(red + 3 * NU * 64 * 16);
+    const int b = blockIdx.x, h = blockIdx.y;
     const int G = a.group;
-    const int h = head / G, n = head - h * G;
-    const int j = threadIdx.x >> 5, c4 = threadIdx.x & 31;
-    uint16_t* op = a.out + (int64_t)b * a.out_stride0 + (int64_t)head * kD + 4 * c4;
-    if ((a.ctx ? a.ctx[b] : a.uniform_len) <= 0) {
-        if (j == 0) *reinterpret_cast<u32x2*>(op) = u32x2{0u, 0u};
+    const int j = threadIdx.x >> 6, c = threadIdx.x & 63;
+    const int nvec = 32 * G;
+    auto load_record = [&](const unsigned char* rec, f32x4 (&v)[NU], float2 (&ml)[NU]) {
+#pragma unroll
+        for (int u = 0; u < NU; ++u) {
+            const int i = c + 64 * u < nvec ? c + 64 * u : 0;
+            v[u] = *reinterpret_cast<const f32x4*>(rec + i * 16);
+            ml[u] = *reinterpret_cast<const float2*>(rec + 512 * G + ((i >> 3) % G) * 8);
+        }
+    };
+    f32x4 v[NU];
+    float2 ml[NU];
+    load_record(a.rec_first + (((int64_t)b * a.num_kv_heads + h) * kFirstPieces + j) * a.rec_stride, v, ml);
+    const int len = a.ctx ? a.ctx[b] : a.uniform_len;
+    const int w0 = a.seg_first[b], w1 = a.seg_last[b];
+    auto store_vec = [&](int i, u32x2 bits) {
+        const int vlane = i >> 3, t = i & 7;
+        uint16_t* op = a.out + (int64_t)b * a.out_stride0 + (int64_t)(h * G + vlane % G) * kD + 16 * t + 4 * (vlane / G);
+        *reinterpret_cast<u32x2*>(op) = bits;
+    };
+    if (len <= 0) {   // no tokens (graph padding): zeros; the piece range of such a row is not written
+        if (j == 0) {
+#pragma unroll
+            for (int u = 0; u < NU; ++u)
+                if (c + 64 * u < nvec) store_vec(c + 64 * u, u32x2{0u, 0u});
+        }
         return;
     }
-    const int w0 = a.seg_first[b], w1 = a.seg_last[b];
-    const int64_t slot0 = (int64_t)h * a.slots_per_head + b;
-    float m = -INFINITY, den = 0.f;
-    f32x4 num = {0.f, 0.f, 0.f, 0.f};
-    for (int wb = w0 + j; wb <= w1; wb += 32) {
-        float2 mlv[4];
-        f32x4 pov[4];
+    const int pieces = w1 - w0 + 1;
+    float m[NU], den[NU];
+    f32x4 num[NU];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int wu = wb + 8 * u <= w1 ? wb + 8 * u : wb;
-            // columns 4 c4 .. 4 c4 + 3 = accumulator tile t = c4 / 4 of lane group g = c4 % 4
-            const unsigned char* rec = a.rec + (slot0 + wu) * a.rec_stride;
-            mlv[u] = *reinterpret_cast<const float2*>(rec + 512 * G + n * 8);
-            pov[u] = *reinterpret_cast<const f32x4*>(rec + (((c4 & 3) * G + n) * 8 + (c4 >> 2)) * 16);
-        }
+    for (int u = 0; u < NU; ++u) {
+        const bool have = j < pieces;
+        m[u] = have ? ml[u].x : -INFINITY;
+        den[u] = have ? ml[u].y : 0.f;
+        num[u] = have ? v[u] : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    for (int k = j + 4; k < pieces; k += 4) {   // pieces beyond the fixed places (kFirstPieces == 4 wavefronts)
+        load_record(a.rec + ((int64_t)h * a.slots_per_head + (w0 + k) + b) * a.rec_stride, v, ml);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            if (wb + 8 * u > w1) break;
-            const float m_new = fmaxf(m, mlv[u].x);
-            const float f_old = __builtin_amdgcn_exp2f(m - m_new);
-            const float f_new = __builtin_amdgcn_exp2f(mlv[u].x - m_new);
-            den = den * f_old + mlv[u].y * f_new;
-            num = num * f_old + pov[u] * f_new;
-            m = m_new;
+        for (int u = 0; u < NU; ++u) {
+            const float mn = fmaxf(m[u], ml[u].x);
+            const float f_old = m[u] == mn ? 1.f : __builtin_amdgcn_exp2f(m[u] - mn);
+            const float f_new = ml[u].x == mn ? 1.f : __builtin_amdgcn_exp2f(ml[u].x - mn);
+            den[u] = den[u] * f_old + ml[u].y * f_new;
+            num[u] = num[u] * f_old + v[u] * f_new;
+            m[u] = mn;
         }
     }
-    red[j][c4][0] = m; red[j][c4][1] = den;
-    red[j][c4][2] = num[0]; red[j][c4][3] = num[1]; red[j][c4][4] = num[2]; red[j][c4][5] = num[3];
-    __syncthreads();
-    if (j == 0) {
-        float mx = m;
+    if (j > 0) {
 #pragma unroll
-        for (int k = 1; k < 8; ++k) mx = fmaxf(mx, red[k][c4][0]);
-        float d_tot = 0.f;
-        f32x4 n_tot = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            const float mk = red[k][c4][0];
-            const float f = mk == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mk - mx);
-            d_tot += red[k][c4][1] * f;
-            n_tot += f32x4{red[k][c4][2], red[k][c4][3], red[k][c4][4], red[k][c4][5]} * f;
+        for (int u = 0; u < NU; ++u) {
+            red_num[((j - 1) * NU + u) * 64 + c] = num[u];
+            red_ml[((j - 1) * NU + u) * 64 + c] = make_float2(m[u], den[u]);
         }
-        const float inv = d_tot > 0.f ? 1.f / d_tot : 0.f;
-        union { __bf16 hv[4]; u32x2 u; } r;
+    }
+    __syncthreads();
+    if (j > 0) return;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) r.hv[e] = (__bf16)(n_tot[e] * inv);
-        *reinterpret_cast<u32x2*>(op) = r.u;
+    for (int u = 0; u < NU; ++u) {
+        for (int w = 0; w < 3; ++w) {
+            const float2 o = red_ml[(w * NU + u) * 64 + c];
+            if (o.y > 0.f) {
+                const float mn = fmaxf(m[u], o.x);
+                const float f_old = m[u] == mn ? 1.f : __builtin_amdgcn_exp2f(m[u] - mn);
+                const float f_new = o.x == mn ? 1.f : __builtin_amdgcn_exp2f(o.x - mn);
+                den[u] = den[u] * f_old + o.y * f_new;
+                num[u] = num[u] * f_old + red_num[(w * NU + u) * 64 + c] * f_new;
+                m[u] = mn;
+            }
+        }
+        if (c + 64 * u < nvec) store_vec(c + 64 * u, pack_out(num[u], den[u] > 0.f ? 1.f / den[u] : 0.f));
     }
 }
 
@@ -988,6 +1036,7 @@ int launch_stream(const DecodeCall& c, const Launch& L, const DecodeWorkspace& w
     a.seg_first = (int32_t*)(base + ws.seg_first_off);
     a.seg_last = (int32_t*)(base + ws.seg_last_off);
     a.rec = (unsigned char*)base + ws.rec_off;
+    a.rec_first = (unsigned char*)base + ws.rec_first_off;
     a.rec_stride = (int)ws.rec_stride;
     a.slots_per_head = (int)ws.slots_per_head;
     a.parts = L.parts;
@@ -1008,14 +1057,20 @@ int launch_merge(void* out, int64_t out_stride0, const int32_t* context_lens, in
     m.ctx = context_lens;
     m.uniform_len = uniform_len > 0 ? 1 : 0;   // only its sign matters here
     m.group = (int)(num_q_heads / num_kv_heads);
+    m.num_kv_heads = (int)num_kv_heads;
     m.slots_per_head = (int)ws.slots_per_head;
     m.seg_first = (const int32_t*)(base + ws.seg_first_off);
     m.seg_last = (const int32_t*)(base + ws.seg_last_off);
     m.rec = (const unsigned char*)base + ws.rec_off;
+    m.rec_first = (const unsigned char*)base + ws.rec_first_off;
     m.rec_stride = (int)ws.rec_stride;
     m.batch = (int)batch;
-    dim3 grid((unsigned)batch, (unsigned)num_q_heads, 1), block(256, 1, 1);
-    hipLaunchKernelGGL(paged_decode_merge_kernel, grid, block, 0, stream, m);
+    dim3 grid((unsigned)batch, (unsigned)num_kv_heads, 1), block(256, 1, 1);
+    const int nu = (32 * m.group + 63) / 64;   // 16-byte vectors of a record per lane
+    if (nu <= 1) hipLaunchKernelGGL(paged_decode_merge_kernel<1>, grid, block, 3 * 1 * 64 * 24, stream, m);
+    else if (nu <= 2) hipLaunchKernelGGL(paged_decode_merge_kernel<2>, grid, block, 3 * 2 * 64 * 24, stream, m);
+    else if (nu <= 4) hipLaunchKernelGGL(paged_decode_merge_kernel<4>, grid, block, 3 * 4 * 64 * 24, stream, m);
+    else hipLaunchKernelGGL(paged_decode_merge_kernel<8>, grid, block, 3 * 8 * 64 * 24, stream, m);
     return (int)hipGetLastError();
 }
 

@@ -167,7 +167,9 @@ __global__ void __launch_bounds__(256) qk_norm_rope_append_kernel(FusedArgs a) {
         // times the weight, rounded: z[i] = pack(z[i].lo * w[2 i], z[i].hi * w[2 i + 1])
         {
             uint32_t t0, t1, t2, t3, t4, t5, t6, t7;
-            __asm__("v_dot2_f32_bf16 %4, %0, %12, 0\n\t"
+            // (volatile: the blocks of a head keep their order, which the DPP reads of the next block count on:
+            // a register written by the vector pipe may be read through DPP two issue slots later)
+            __asm__ volatile("v_dot2_f32_bf16 %4, %0, %12, 0\n\t"
                     "v_dot2_f32_bf16 %5, %0, %16, 0\n\t"
                     "v_dot2_f32_bf16 %6, %1, %13, 0\n\t"
                     "v_dot2_f32_bf16 %7, %1, %17, 0\n\t"
@@ -191,7 +193,7 @@ __global__ void __launch_bounds__(256) qk_norm_rope_append_kernel(FusedArgs a) {
         const uint32_t ones = 0x3f803f80u;
         auto rotate2 = [&](int i, uint32_t& o0, uint32_t& o1) {
             uint32_t p0, p1, t0, t1, t2, t3, t4, t5, t6, t7;
-            __asm__("v_mov_b32_dpp %2, %12 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+            __asm__ volatile("v_mov_b32_dpp %2, %12 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
                     "v_mov_b32_dpp %3, %13 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
                     "v_dot2_f32_bf16 %4, %12, %14, 0\n\t"
                     "v_dot2_f32_bf16 %5, %2, %16, 0\n\t"
