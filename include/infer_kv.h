@@ -37,6 +37,8 @@ extern "C" {
 #define INFER_KV_ESTATE       -5   /* block pool: the call violates an invariant the reference
                                       asserts (double allocate, out of blocks, ...); see
                                       infer_pool_last_error()                                   */
+#define INFER_KV_EBUSY        -7   /* the library's own scratch array is still in use by work
+                                      pending on another stream (infer_paged_decode_noalloc_bf16) */
 #define INFER_KV_ENOTINIT     -6   /* first decode call on this device made while its stream is
                                       being captured: call infer_kv_init() before the capture    */
 
@@ -214,8 +216,10 @@ int infer_paged_decode_uniform_bf16(const void* q, int64_t q_stride0,
  * Hkv * (CUs * 4 / Hkv + batch) * 520 * G bytes, i.e. 3.2 MB at batch 64, Hq/Hkv = 32/8 and 4.5 MB at
  * batch 8, 64/8 on 256 compute units, against the INFER_KV_DECODE_NOALLOC_SCRATCH_BYTES of the array.
  * The array keeps the last call's contents and needs no clearing (every record that is read was
- * written by the same call).  All calls on one GPU share it: calls that overlap on one GPU (two
- * streams, two threads) race; calls ordered on one stream are safe.  The address of the array is
+ * written by the same call).  All calls on one GPU share it: calls ordered on one stream are safe; a
+ * call on another stream than the previous one is refused with INFER_KV_EBUSY while that stream still
+ * has work pending (a cheap host-side check; calls racing on two host threads, and a capture that will
+ * be replayed beside other users of the array, remain the caller's to order).  The address of the array is
  * resolved by infer_kv_init() or by the first decode call on the device outside stream capture. */
 #define INFER_KV_DECODE_NOALLOC_SCRATCH_BYTES ((size_t)16 << 20)
 int infer_paged_decode_noalloc_bf16(const void* q, int64_t q_stride0,

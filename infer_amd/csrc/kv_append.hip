@@ -207,6 +207,7 @@ const char* infer_kv_strerror(int code) {
         case INFER_KV_EWORKSPACE: return "workspace too small";
         case INFER_KV_EUNSUPPORTED: return "shape not built (head_dim must be 128, group size <= 16, block_size % 32 == 0)";
         case INFER_KV_ESTATE: return "block pool invariant violated (see infer_pool_last_error)";
+        case INFER_KV_EBUSY: return "the library's scratch array is in use by work pending on another stream";
         case INFER_KV_ENOTINIT: return "first decode call on this device under stream capture: call infer_kv_init() first";
         default: break;
     }

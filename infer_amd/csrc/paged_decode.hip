@@ -866,6 +866,8 @@ namespace {
 struct DeviceState {
     int cus;          // compute units
     void* scratch;    // device address of infer_kv_decode_scratch on this device
+    hipStream_t last_scratch_stream;   // stream of the last call that used the scratch array
+    bool scratch_used;
 };
 DeviceState g_dev[kMaxDevices];
 bool g_dev_known[kMaxDevices] = {false};
@@ -874,7 +876,7 @@ bool g_dev_known[kMaxDevices] = {false};
 // address of the scratch array.  Two first calls that race do the same work twice and store the same
 // values.  A first call that arrives while `stream` is being captured is refused: the set-up calls
 // are not stream work and must not run inside a capture.
-int init_device(hipStream_t stream, bool have_stream, const DeviceState** out) {
+int init_device(hipStream_t stream, bool have_stream, DeviceState** out) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return (int)e;
@@ -895,6 +897,8 @@ int init_device(hipStream_t stream, bool have_stream, const DeviceState** out) {
         e = hipFuncSetAttribute((const void*)paged_decode_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 8 * kLdsPerWave);
         if (e != hipSuccess) return (int)e;
         d.scratch = nullptr;
+        d.last_scratch_stream = nullptr;
+        d.scratch_used = false;
         e = hipGetSymbolAddress(&d.scratch, HIP_SYMBOL(infer_kv_decode_scratch));
         if (e != hipSuccess) return (int)e;
         if (d.scratch == nullptr) return INFER_KV_EINVAL;
@@ -1112,7 +1116,7 @@ int infer_paged_decode_split_bf16(const void* q, int64_t q_stride0, const void* 
     if (rc) return rc;
     const DecodeWorkspace ws = decode_workspace_layout(batch, num_q_heads / num_kv_heads, num_kv_heads);
     if (ws.total_bytes > workspace_bytes) return INFER_KV_EWORKSPACE;
-    const DeviceState* dev = nullptr;
+    DeviceState* dev = nullptr;
     rc = init_device((hipStream_t)stream, true, &dev);
     if (rc) return rc;
     Launch L;
@@ -1155,7 +1159,7 @@ int infer_paged_decode_bf16(const void* q, int64_t q_stride0, const void* k_cach
     if (rc) return rc;
     const DecodeWorkspace ws = decode_workspace_layout(batch, num_q_heads / num_kv_heads, num_kv_heads);
     if (ws.total_bytes > workspace_bytes) return INFER_KV_EWORKSPACE;
-    const DeviceState* dev = nullptr;
+    DeviceState* dev = nullptr;
     rc = init_device((hipStream_t)stream, true, &dev);
     if (rc) return rc;
     Launch L;
@@ -1180,7 +1184,7 @@ int infer_paged_decode_uniform_bf16(const void* q, int64_t q_stride0, const void
     if (rc) return rc;
     const DecodeWorkspace ws = decode_workspace_layout(batch, num_q_heads / num_kv_heads, num_kv_heads);
     if (ws.total_bytes > workspace_bytes) return INFER_KV_EWORKSPACE;
-    const DeviceState* dev = nullptr;
+    DeviceState* dev = nullptr;
     rc = init_device((hipStream_t)stream, true, &dev);
     if (rc) return rc;
     Launch L;
@@ -1212,10 +1216,26 @@ int infer_paged_decode_noalloc_bf16(const void* q, int64_t q_stride0, const void
     if (rc) return rc;
     rc = check_out(out, out_stride0, num_q_heads);
     if (rc) return rc;
-    const DeviceState* dev = nullptr;
+    DeviceState* dev = nullptr;
     rc = init_device((hipStream_t)stream, true, &dev);
     if (rc) return rc;
     void* scratch = dev->scratch;
+    // All calls on a device share the scratch array.  A call on another stream than the last one, while
+    // that stream still has work pending, would overwrite records in use: refused (a cheap check, not a
+    // lock: calls that race on two host threads are still the caller's to order).  Streams under capture
+    // are not queried.
+    {
+        const hipStream_t st = (hipStream_t)stream;
+        hipStream_t last = __atomic_load_n(&dev->last_scratch_stream, __ATOMIC_ACQUIRE);
+        if (__atomic_load_n(&dev->scratch_used, __ATOMIC_ACQUIRE) && last != st) {
+            hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+            const bool capturing = hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone;
+            if (!capturing && hipStreamQuery(last) == hipErrorNotReady) return INFER_KV_EBUSY;
+            (void)hipGetLastError();
+        }
+        __atomic_store_n(&dev->last_scratch_stream, st, __ATOMIC_RELEASE);
+        __atomic_store_n(&dev->scratch_used, true, __ATOMIC_RELEASE);
+    }
     Launch L;
     rc = plan_launch(num_kv_heads, /*split_workgroups=*/0, dev->cus, INFER_KV_DECODE_PARTS, &L);
     if (rc) return rc;

@@ -90,3 +90,24 @@ def test_replays_inside_a_hip_graph(gpu):
         assert _call("workspace", wl, want, ws) == 0                     # eager work between the replays
         torch.cuda.synchronize()
         assert np.array_equal(bits(out), bits(want)), wl.name
+
+
+def test_another_stream_is_refused_while_the_last_one_is_busy(gpu):
+    """All calls on a GPU share the library's scratch array: a call on another stream than the previous one
+    is refused while that stream still has work pending, and accepted once it has drained."""
+    wl = workloads.make_decode_workload("na-busy", [900, 70, 300], 32, 8, seed=25).to(gpu)
+    out_a, out_b = torch.empty_like(wl.q), torch.empty_like(wl.q)
+    sa, sb = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(sa):
+        assert _call("noalloc", wl, out_a) == 0
+        torch.cuda._sleep(400_000_000)            # keeps stream A busy for a fraction of a second
+    with torch.cuda.stream(sb):
+        assert _call("noalloc", wl, out_b) == -7  # INFER_KV_EBUSY: nothing was enqueued
+    sa.synchronize()
+    with torch.cuda.stream(sb):
+        assert _call("noalloc", wl, out_b) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(out_a), bits(out_b))
+    assert _call("noalloc", wl, out_b) == 0       # back on the default stream, everything drained
+    torch.cuda.synchronize()
