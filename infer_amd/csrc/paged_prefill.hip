@@ -57,6 +57,7 @@ struct PrefillArgs {
     int block_size;
     int num_blocks;
     int max_sk;             // paged keys: what a block-table row can address (table_cols * block_size)
+    int table_cols;         // entries of a block-table row
     float scale_log2;
     int causal;
 };
@@ -139,6 +140,17 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     const int head = kvh * a.group + (block_z % parts) * kHeads + (QB == 1 ? wave : wave % kHeads);
     const int qb = QB == 1 ? 0 : wave / kHeads;            // query block of this wavefront inside the workgroup
 
+    // The first kTblLds block ids of the sequence go to LDS (see below).  Their loads depend on nothing but
+    // the sequence index, so they are issued first and travel while the sequence bounds are fetched;
+    // entries of the row behind the sequence's own blocks are loaded too and never used.
+    constexpr int kTblPer = (kTblLds + 64 * WAVES - 1) / (64 * WAVES);
+    const int tbl_cols = a.bt ? (a.table_cols < kTblLds ? a.table_cols : kTblLds) : 0;
+    int tbl_reg[kTblPer];
+#pragma unroll
+    for (int i = 0; i < kTblPer; ++i) {
+        const int c = tid + i * 64 * WAVES;
+        tbl_reg[i] = c < tbl_cols ? a.bt[(int64_t)b * a.bt_stride0 + c] : 0;
+    }
     const int q_beg = a.cu_q[b], q_end = a.cu_q[b + 1];
     const int k_beg = a.cu_k[b], k_end = a.cu_k[b + 1];
     const int sq = q_end - q_beg;
@@ -177,6 +189,23 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     const int nsteps = (key_end_of(wg_q0, QB * kQBlock) + kStep - 1) / kStep;
     const int my_steps = live ? (key_end_of(q0, kQBlock) + kStep - 1) / kStep : 0;
 
+    // The first kTblLds block ids of the sequence are copied to LDS behind the ring (one barrier, before
+    // anything is fetched): a lookup in memory, behind a division by the block size, would put some
+    // 300 ns of dependent work in front of every tile fetch, and a register copy gets spilled, whose
+    // reload is a vector load and so drains the ring.  Tiles are fetched in order, so the block index
+    // and the step inside the block are counters.
+    const int steps_per_blk = a.block_size / kStep;
+    int* lds_tbl = reinterpret_cast<int*>(lds_all + kRing * kTileBytes);
+    if (a.bt) {
+#pragma unroll
+        for (int i = 0; i < kTblPer; ++i) {
+            const int c = tid + i * 64 * WAVES;
+            if (c < tbl_cols) lds_tbl[c] = tbl_reg[i];
+        }
+        __syncthreads();
+    }
+    // (the loads of Q are issued after this wait, not before it: the compiler's wait for the block ids
+    // would wait for them as well)
     bf16x8 qreg[kNQ][4];
     bf16x8 ones;
 #pragma unroll
@@ -244,19 +273,6 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         ld_off[i] = (uint32_t)(ld_key(i) * tok_stride) + ld_col(i);       // < 2^30: tok_stride < 2^24, 32 rows
         ld_dst[i] = (L >> 3) * kKTileBytes + (L & 7) * kGroupB;
     }
-    // The first kTblLds block ids of the sequence are copied to LDS behind the ring (one barrier, before
-    // anything is fetched): a lookup in memory, behind a division by the block size, would put some
-    // 300 ns of dependent work in front of every tile fetch, and a register copy gets spilled, whose
-    // reload is a vector load and so drains the ring.  Tiles are fetched in order, so the block index
-    // and the step inside the block are counters.
-    const int steps_per_blk = a.block_size / kStep;
-    int* lds_tbl = reinterpret_cast<int*>(lds_all + kRing * kTileBytes);
-    if (a.bt) {
-        const int nblk = (nsteps + steps_per_blk - 1) / steps_per_blk;
-        const int32_t* row = a.bt + (int64_t)b * a.bt_stride0;
-        for (int i = tid; i < nblk && i < kTblLds; i += 64 * WAVES) lds_tbl[i] = row[i];
-        __syncthreads();
-    }
     int f_blk = 0, f_in = 0;      // block index and step inside it of the next tile to fetch
     int64_t f_base = 0;           // element offset of that block
     auto fetch = [&](int s, int buf) {
@@ -308,12 +324,14 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     // tile s lives in ring buffer s % 3: requested at the top of step s - 2, landed (own loads counted,
     // then the barrier) at the end of step s - 1, read during step s; the buffer is requested again at
     // the top of step s + 1, after the barrier that ends step s.
-    // Q and the block ids have arrived before the first transfer is issued: the compiler does not see
-    // the transfers, so any wait of its own for these earlier loads inside the loop would be a wait for
-    // zero outstanding loads and drain the ring.
-    landed_all();
+    // The loads of Q are still in flight when the first two tiles are requested, so that the two round
+    // trips to memory overlap; one wait for everything follows.  It is written out, although the
+    // compiler would wait for Q by itself: the compiler does not see the transfers, so its own wait
+    // would sit at the first use of Q inside the loop, as a wait for zero outstanding loads in every
+    // step, which drains the ring.
     fetch(0, 0);
-    if (nsteps > 1) { fetch(1, 1); landed_but_newest(); } else { landed_all(); }
+    if (nsteps > 1) fetch(1, 1);
+    landed_all();
     __syncthreads();
 
     auto step = [&](int s, int buf) {
@@ -471,6 +489,7 @@ extern "C" int infer_paged_prefill_bf16(const void* q, int64_t q_stride0, const 
     a.group = G;
     a.block_size = (int)block_size; a.num_blocks = (int)num_blocks;
     a.max_sk = block_table ? (int)(table_cols * block_size) : 0x7fffffff;
+    a.table_cols = block_table ? (int)table_cols : 0;
     a.scale_log2 = scale * 1.4426950408889634f;
     a.causal = causal ? 1 : 0;
     hipStream_t st = (hipStream_t)stream;
