@@ -128,12 +128,20 @@ __device__ __forceinline__ int wave_sum(int x) { return __builtin_amdgcn_readlan
 __device__ __forceinline__ float max_xor16(float x) {
     const unsigned u = __builtin_bit_cast(unsigned, x);
     const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-    return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+    // the halves go through scalars of their own: a bit cast applied to `r[1]` itself reads element 0
+    const unsigned lo = r[0], hi = r[1];
+    float m;   // written out: fmaxf would first quiet a NaN in each operand, two more instructions
+    __asm__("v_max_f32_e32 %0, %1, %2" : "=v"(m) : "v"(lo), "v"(hi));
+    return m;
 }
 __device__ __forceinline__ float max_xor32(float x) {
     const unsigned u = __builtin_bit_cast(unsigned, x);
     const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+    // the halves go through scalars of their own: a bit cast applied to `r[1]` itself reads element 0
+    const unsigned lo = r[0], hi = r[1];
+    float m;   // written out: fmaxf would first quiet a NaN in each operand, two more instructions
+    __asm__("v_max_f32_e32 %0, %1, %2" : "=v"(m) : "v"(lo), "v"(hi));
+    return m;
 }
 
 // Keeps the compiler from moving LDS traffic across this point.  The LDS queue of one

@@ -20,6 +20,7 @@
 // LDS store instructions; tile s + 2 is in flight while tile s + 1 has landed and tile s is consumed;
 // one barrier per step).  Without staging registers the kernel fits three wavefronts per SIMD.
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include <stdint.h>
 
 
@@ -74,12 +75,20 @@ __device__ __forceinline__ void lds_order() { __asm__ volatile("" ::: "memory");
 __device__ __forceinline__ float max_xor16(float x) {
     const unsigned u = __builtin_bit_cast(unsigned, x);
     const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-    return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+    // the halves go through scalars of their own: a bit cast applied to `r[1]` itself reads element 0
+    const unsigned lo = r[0], hi = r[1];
+    float m;   // written out: fmaxf would first quiet a NaN in each operand, two more instructions
+    __asm__("v_max_f32_e32 %0, %1, %2" : "=v"(m) : "v"(lo), "v"(hi));
+    return m;
 }
 __device__ __forceinline__ float max_xor32(float x) {
     const unsigned u = __builtin_bit_cast(unsigned, x);
     const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+    // the halves go through scalars of their own: a bit cast applied to `r[1]` itself reads element 0
+    const unsigned lo = r[0], hi = r[1];
+    float m;   // written out: fmaxf would first quiet a NaN in each operand, two more instructions
+    __asm__("v_max_f32_e32 %0, %1, %2" : "=v"(m) : "v"(lo), "v"(hi));
+    return m;
 }
 
 // LDS layout of a tile.  Key k of the step is row  16 ((k >> 2) & 1) + 4 (k >> 3) + (k & 3)  of the
@@ -250,8 +259,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     // Address = uniform 64-bit base (scalar registers) + per-lane 32-bit byte offset: no vector
     // arithmetic per transfer.
     typedef __attribute__((address_space(3))) void* lptr_t;
-    auto dma16 = [&](const uint16_t* base, uint32_t byte_off, unsigned char* dst) {
-        const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)dst;
+    auto dma16 = [&](const unsigned char* base, uint32_t byte_off, uint32_t lds_addr) {
         __asm__ volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                          :: "v"(byte_off), "s"(base), "s"(lds_addr) : "memory", "m0");
     };
@@ -260,7 +268,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     // loads 0 .. 7 are the K tile, 8 .. 15 the V tile: with four wavefronts (load w + 4 i) that is a
     // matter of i alone
     auto load_is_k = [&](int i) { return WAVES == 4 ? i < 2 : (wave + i * WAVES < 16 ? wave + i * WAVES : 0) < 8; };
-    uint32_t ld_off[kLoads];                      // element offset inside a tile of what this lane fetches
+    uint32_t ld_byte[kLoads];                     // byte offset inside a tile of what this lane fetches
     int ld_dst[kLoads];                           // LDS byte offset of the load inside a tile pair (uniform)
     auto ld_key = [&](int i) {                    // key (row of the tile in memory) of load i of this lane:
         const int L = wave + i * WAVES < 16 ? wave + i * WAVES : 0;
@@ -270,43 +278,49 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
         const int L = wave + i * WAVES < 16 ? wave + i * WAVES : 0;
-        ld_off[i] = (uint32_t)(ld_key(i) * tok_stride) + ld_col(i);       // < 2^30: tok_stride < 2^24, 32 rows
+        ld_byte[i] = 2 * ((uint32_t)(ld_key(i) * tok_stride) + ld_col(i));   // < 2^31: tok_stride < 2^24, 32 rows
         ld_dst[i] = (L >> 3) * kKTileBytes + (L & 7) * kGroupB;
     }
-    int f_blk = 0, f_in = 0;      // block index and step inside it of the next tile to fetch
-    int64_t f_base = 0;           // element offset of that block
-    auto fetch = [&](int s, int buf) {
-        const int tok0 = s * kStep;
-        int64_t base;
+    // Tiles are fetched in order, so the address of the next one is a running 64-bit byte offset: one
+    // addition per tile, a table lookup and a multiplication only where a block begins.  (A step of a
+    // wavefront is some 250 instructions issued in order; address arithmetic redone from the step index
+    // was 40 scalar instructions of them.)
+    const int64_t tile_bytes = 2 * (int64_t)kStep * a.tok_stride;
+    int64_t f_byte = a.bt ? 0 : 2 * (int64_t)k_beg * a.tok_stride;   // byte offset of the next tile to fetch
+    int f_blk = 0, f_left = 0;    // next block of the table, tiles left in the current one
+    const int whole_tiles = sk / kStep;                        // tiles in front of this index are whole
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(lptr_t)lds_all;
+    uint32_t ld_lds[kLoads];                                   // LDS address of load i in ring buffer 0 (uniform)
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) ld_lds[i] = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)ld_dst[i]);
+    // ring_off: byte offset of the ring buffer that takes the tile
+    auto fetch = [&](int s, int ring_off) {
         if (a.bt) {
-            if (f_in == 0) {
+            if (f_left == 0) {
                 int blk;
                 if (f_blk < kTblLds) blk = __builtin_amdgcn_readfirstlane(lds_tbl[f_blk]);
                 else blk = __builtin_amdgcn_readfirstlane(a.bt[(int64_t)b * a.bt_stride0 + f_blk]);   // drains the ring
                 blk = blk < 0 ? 0 : (blk >= a.num_blocks ? a.num_blocks - 1 : blk);
-                f_base = (int64_t)blk * a.blk_stride;
+                f_byte = 2 * (int64_t)blk * a.blk_stride;
+                f_left = steps_per_blk;
+                ++f_blk;
             }
-            base = f_base + (int64_t)(f_in * kStep) * a.tok_stride;
-            if (++f_in == steps_per_blk) { f_in = 0; ++f_blk; }
-        } else {
-            base = ((int64_t)k_beg + tok0) * a.tok_stride;
+            --f_left;
         }
-        const uint16_t* kp = a.k + base;
-        const uint16_t* vp = a.v + base;
-        unsigned char* dst = lds_all + buf * kTileBytes;
-        if (tok0 + kStep <= sk) {
+        const unsigned char* kp = reinterpret_cast<const unsigned char*>(a.k) + f_byte;
+        const unsigned char* vp = reinterpret_cast<const unsigned char*>(a.v) + f_byte;
+        f_byte += tile_bytes;
+        if (s < whole_tiles) {
 #pragma unroll
-            for (int i = 0; i < kLoads; ++i) {
-                dma16(load_is_k(i) ? kp : vp, 2 * ld_off[i], dst + ld_dst[i]);
-            }
+            for (int i = 0; i < kLoads; ++i) dma16(load_is_k(i) ? kp : vp, ld_byte[i], ld_lds[i] + (uint32_t)ring_off);
         } else {
             // rows past the end of the sequence (last step only) re-read its last row: finite data whose
             // probabilities are masked to zero, instead of whatever lies behind the sequence
-            const int last = sk - 1 - tok0;
+            const int last = sk - 1 - s * kStep;
 #pragma unroll
             for (int i = 0; i < kLoads; ++i) {
                 const int r = ld_key(i) < last ? ld_key(i) : last;
-                dma16(load_is_k(i) ? kp : vp, 2 * ((uint32_t)(r * tok_stride) + ld_col(i)), dst + ld_dst[i]);
+                dma16(load_is_k(i) ? kp : vp, 2 * ((uint32_t)(r * tok_stride) + ld_col(i)), ld_lds[i] + (uint32_t)ring_off);
             }
         }
     };
@@ -330,14 +344,18 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     // would sit at the first use of Q inside the loop, as a wait for zero outstanding loads in every
     // step, which drains the ring.
     fetch(0, 0);
-    if (nsteps > 1) fetch(1, 1);
+    if (nsteps > 1) fetch(1, kTileBytes);
     landed_all();
     __syncthreads();
 
-    auto step = [&](int s, int buf) {
-        const int buf2 = buf == 0 ? 2 : buf - 1;          // (s + 2) % 3
-        if (s + 2 < nsteps) fetch(s + 2, buf2);
-        const unsigned char* kb = lds_all + buf * kTileBytes;
+    // With four wavefronts the loop is unrolled by the ring, so that the buffer of tile s is a constant of
+    // each copy and every LDS address of the step is a per-lane register plus an immediate.
+    // ring: byte offset of the buffer that holds tile s; ring_next: of the one that takes tile s + 2
+    // (plain integers, or compile-time constants in the unrolled loop)
+    auto step = [&](int s, auto ring_v, auto ring_next_v) {
+        const int ring = ring_v, ring_next = ring_next_v;
+        if (s + 2 < nsteps) fetch(s + 2, ring_next);
+        const unsigned char* kb = lds_all + ring;
         const int tok0 = s * kStep;
 
         if (QB == 1 || s < my_steps) {   // wavefronts whose queries end earlier skip the keys they cannot see
@@ -414,7 +432,26 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         if (s + 2 < nsteps) landed_but_newest(); else landed_all();
         __syncthreads();
     };
-    for (int s = 0, buf = 0; s < nsteps; ++s, buf = buf == 2 ? 0 : buf + 1) step(s, buf);
+    if constexpr (WAVES == 4) {
+        using B0 = std::integral_constant<int, 0>;
+        using B1 = std::integral_constant<int, kTileBytes>;
+        using B2 = std::integral_constant<int, 2 * kTileBytes>;
+        int s = 0;
+        for (; s + 2 < nsteps; s += 3) {
+            step(s, B0{}, B2{});
+            step(s + 1, B1{}, B0{});
+            step(s + 2, B2{}, B1{});
+        }
+        if (s < nsteps) step(s, B0{}, B2{});
+        if (s + 1 < nsteps) step(s + 1, B1{}, B0{});
+    } else {
+        // three wavefronts issue six transfers each: the unrolled form runs out of registers
+        for (int s = 0, ring = 0, ring_next = 2 * kTileBytes; s < nsteps; ++s) {
+            step(s, ring, ring_next);
+            ring_next = ring;                                            // (s + 3) % 3 = s % 3
+            ring = ring == 2 * kTileBytes ? 0 : ring + kTileBytes;
+        }
+    }
 
     if (!live) return;
 #pragma unroll

@@ -101,6 +101,29 @@ def test_equal_keys_give_mean_of_values(gpu):
         assert np.abs(got[i] - np.repeat(mean, 2, axis=0)).max() <= 1e-2
 
 
+def test_row_maximum_covers_every_key_of_a_step(gpu):
+    """One key whose score lies some 350 log2 units above all others, once at each of the 32 positions of
+    a step: the softmax gives it weight 1 wherever it sits.  A running maximum taken over part of a step
+    only (say, the keys one row of lanes holds) leaves the exponential of that key to overflow."""
+    lens = [96] * 32
+    wl = workloads.make_decode_workload("spike", lens, 16, 8, seed=11).to(gpu)
+    g = wl.num_q_heads // wl.num_kv_heads
+    for i in range(32):
+        pos = 32 + i                                                     # the second of three steps
+        blk = int(wl.block_table[i, pos // wl.block_size])
+        q0 = wl.q[i, ::g].float()                                        # first query head of every KV head
+        c = 250.0 / (wl.scale * (q0 * q0).sum(dim=-1, keepdim=True))     # score * scale = 250 for that head
+        wl.k_cache[blk, pos % wl.block_size] = (c * q0).to(torch.bfloat16)
+    got = f32(gpu_decode(wl))
+    want = oracle_decode(wl)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= ATTN_ATOL
+    for i in range(32):                                                  # weight 1: the key's value row, bit for bit
+        pos = 32 + i
+        blk = int(wl.block_table[i, pos // wl.block_size])
+        assert np.array_equal(got[i, ::g], f32(wl.v_cache[blk, pos % wl.block_size]))
+
+
 def test_block_permutation_invariance(gpu):
     """Same logical tokens under a different physical placement give bit-identical output."""
     wl = workloads.make_decode_workload("perm", [700, 1023, 40], 32, 8, nblk=32, seed=7).to(gpu)

@@ -47,6 +47,28 @@ def test_small_shapes_with_and_without_prefix(gpu, hq, hkv):
     assert np.abs(f32(out) - oracle_paged(wl, kc, vc)).max() <= ATTN_ATOL
 
 
+def test_row_maximum_covers_every_key_of_a_step(gpu):
+    """One key per prompt whose score lies some 350 log2 units above all others, at each of the 32
+    positions of a step in turn: every query behind it gives it weight 1.  A running maximum taken over
+    part of a step only leaves the exponential of that key to overflow."""
+    n = 32
+    wl = workloads.make_prefill_workload("spike", [96] * n, [0] * n, 16, 8, seed=12, pad_fraction=0.0).to(gpu)
+    g = wl.num_q_heads // wl.num_kv_heads
+    for j in range(n):
+        rows = slice(96 * j, 96 * (j + 1))
+        wl.q[rows] = wl.q[96 * j]                                        # one query vector per head for the whole prompt
+        q0 = wl.q[96 * j, ::g].float()
+        c = 250.0 / (wl.scale * (q0 * q0).sum(dim=-1, keepdim=True))
+        wl.k_new[96 * j + 32 + j] = (c * q0).to(torch.bfloat16)           # key 32 + j of prompt j
+    out, kc, vc = run_paged(wl)
+    got, want = f32(out), oracle_paged(wl, kc, vc)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= ATTN_ATOL
+    for j in range(n):                                                   # queries at and behind the key return its value row
+        p = 96 * j + 32 + j
+        assert np.array_equal(got[p:96 * (j + 1), ::g], np.broadcast_to(f32(wl.v_new[p]), (96 * (j + 1) - p, 8, 128)))
+
+
 @pytest.mark.parametrize("bs", [32, 64, 512])
 def test_block_sizes(gpu, bs):
     wl = workloads.make_prefill_workload("p", [70, 200, 5], [bs if bs <= 64 else 0, 0, 0], 16, 8, bs=bs, seed=bs,
