@@ -232,12 +232,12 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     // query (one MFMA per tile and step instead of eight vector adds), of the same bf16 values the
     // numerator is built from; all four accumulator rows of a lane hold the same sum.
     f32x4 lacc[kNQ];
-    float m_run[kNQ];
+    float m_neg[kNQ];
 #pragma unroll
     for (int u = 0; u < kNQ; ++u) {
 #pragma unroll
         for (int t = 0; t < 8; ++t) acc[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-        m_run[u] = -INFINITY;
+        m_neg[u] = INFINITY;
         lacc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
@@ -352,9 +352,12 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     // each copy and every LDS address of the step is a per-lane register plus an immediate.
     // ring: byte offset of the buffer that holds tile s; ring_next: of the one that takes tile s + 2
     // (plain integers, or compile-time constants in the unrolled loop)
-    auto step = [&](int s, auto ring_v, auto ring_next_v) {
+    // inner_tag: a step of the main loop, which is known to request tile s + 2 and to lie in front of the
+    // diagonal of every wavefront: no branch for either
+    auto step = [&](int s, auto ring_v, auto ring_next_v, auto inner_tag) {
+        constexpr bool kInner = decltype(inner_tag)::value;
         const int ring = ring_v, ring_next = ring_next_v;
-        if (s + 2 < nsteps) fetch(s + 2, ring_next);
+        if (kInner || s + 2 < nsteps) fetch(s + 2, ring_next);
         const unsigned char* kb = lds_all + ring;
         const int tok0 = s * kStep;
 
@@ -387,7 +390,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) sv[4 * t + e] = sc[u][t][e];
-            if (tok0 + kStep - 1 > lim_lo[u]) {      // wave-uniform: off the diagonal no lane masks anything
+            if (!kInner && tok0 + kStep - 1 > lim_lo[u]) {      // wave-uniform: off the diagonal no lane masks anything
                 // key tok0 + 8 g + i is masked iff i > rel; written so that nothing but this one
                 // subtraction could be computed ahead of the branch
                 const int rel = my_limit[u] - tok0 - 8 * g;
@@ -400,18 +403,20 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
             for (int i = 1; i < 8; ++i) mx = fmaxf(mx, sv[i]);
             mx = max_xor32(max_xor16(mx));
             mx *= a.scale_log2;                                  // scale > 0: the maximum commutes with it
-            const bool grow = mx > m_run[u] + kLazy;             // -inf + kLazy = -inf: the first finite maximum always grows
+            // m_neg is minus the running maximum, +inf before the first step: key 0 is visible to every
+            // query, so step 0 always "grows" (inf > kLazy) and sets it.  (A query without any visible key,
+            // sq > sk, keeps +inf; its row is written as zeros at the end.)
+            const bool grow = mx + m_neg[u] > kLazy;
             if (__any(grow)) {
-                const float alpha = grow ? __builtin_amdgcn_exp2f(m_run[u] - mx) : 1.f;
-                m_run[u] = grow ? mx : m_run[u];
+                const float alpha = grow ? __builtin_amdgcn_exp2f(-m_neg[u] - mx) : 1.f;
+                m_neg[u] = grow ? -mx : m_neg[u];
                 lacc[u] *= alpha;
 #pragma unroll
                 for (int t = 0; t < 8; ++t) acc[u][t] *= alpha;
             }
-            const float m_neg = m_run[u] == -INFINITY ? 0.f : -m_run[u];
 #pragma unroll
             for (int i = 0; i < 8; ++i)
-                pb[u][i] = (__bf16)__builtin_amdgcn_exp2f(__builtin_fmaf(sv[i], a.scale_log2, m_neg));
+                pb[u][i] = (__bf16)__builtin_amdgcn_exp2f(__builtin_fmaf(sv[i], a.scale_log2, m_neg[u]));
             lacc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb[u], lacc[u], 0, 0, 0);
         }
 
@@ -429,25 +434,37 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
         }
 
         // tile s + 1 must be in LDS for everybody: own loads first, then the barrier
-        if (s + 2 < nsteps) landed_but_newest(); else landed_all();
+        if (kInner || s + 2 < nsteps) landed_but_newest(); else landed_all();
         __syncthreads();
     };
+    // steps in front of inner_end request a tile two steps ahead and end in front of the keys the
+    // workgroup's first query cannot see (the earliest diagonal of the workgroup)
+    const int wg_lim_lo = a.causal ? (wg_q0 + shift < sk - 1 ? wg_q0 + shift : sk - 1) : sk - 1;
+    const int free_steps = wg_lim_lo >= 0 ? (wg_lim_lo + 1) / kStep : 0;
+    const int inner_end = nsteps - 2 < free_steps ? nsteps - 2 : free_steps;
+    using Inner = std::true_type;
+    using Outer = std::false_type;
     if constexpr (WAVES == 4) {
         using B0 = std::integral_constant<int, 0>;
         using B1 = std::integral_constant<int, kTileBytes>;
         using B2 = std::integral_constant<int, 2 * kTileBytes>;
         int s = 0;
-        for (; s + 2 < nsteps; s += 3) {
-            step(s, B0{}, B2{});
-            step(s + 1, B1{}, B0{});
-            step(s + 2, B2{}, B1{});
+        for (; s + 2 < inner_end; s += 3) {
+            step(s, B0{}, B2{}, Inner{});
+            step(s + 1, B1{}, B0{}, Inner{});
+            step(s + 2, B2{}, B1{}, Inner{});
         }
-        if (s < nsteps) step(s, B0{}, B2{});
-        if (s + 1 < nsteps) step(s + 1, B1{}, B0{});
+        for (; s + 2 < nsteps; s += 3) {
+            step(s, B0{}, B2{}, Outer{});
+            step(s + 1, B1{}, B0{}, Outer{});
+            step(s + 2, B2{}, B1{}, Outer{});
+        }
+        if (s < nsteps) step(s, B0{}, B2{}, Outer{});
+        if (s + 1 < nsteps) step(s + 1, B1{}, B0{}, Outer{});
     } else {
         // three wavefronts issue six transfers each: the unrolled form runs out of registers
         for (int s = 0, ring = 0, ring_next = 2 * kTileBytes; s < nsteps; ++s) {
-            step(s, ring, ring_next);
+            step(s, ring, ring_next, Outer{});
             ring_next = ring;                                            // (s + 3) % 3 = s % 3
             ring = ring == 2 * kTileBytes ? 0 : ring + kTileBytes;
         }
@@ -458,6 +475,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     for (int u = 0; u < kNQ; ++u) {
         const float l = lacc[u][0];
         if (my_q[u] < sq) {
+            const bool none = my_limit[u] < 0;          // no key visible to this query (sq > sk): zeros, whatever the sums hold
             const float inv = l > 0.f ? 1.f / l : 0.f;
             uint16_t* op = a.out + (int64_t)(q_beg + my_q[u]) * a.out_stride0 + (int64_t)head * kD + 4 * g;
 #pragma unroll
@@ -465,7 +483,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
                 union { __bf16 hv[4]; u32x2 w; } r;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) r.hv[e] = (__bf16)(acc[u][t][e] * inv);
-                *reinterpret_cast<u32x2*>(op + 16 * t) = r.w;
+                *reinterpret_cast<u32x2*>(op + 16 * t) = none ? u32x2{0u, 0u} : r.w;
             }
         }
     }

@@ -238,6 +238,32 @@ def test_more_keys_than_queries_is_bottom_right_aligned(gpu):
     assert (out[-1].float().cpu().view(8, 2, 128) - ref).abs().max() <= ATTN_ATOL
 
 
+def test_more_queries_than_keys_gives_zero_rows_without_a_visible_key(gpu):
+    """sq > sk (outside what the engine produces, since every query's own key is in the cache): with the
+    bottom-right alignment the first sq - sk queries see no key at all.  Their rows are zeros (what
+    flash-attn documents for a fully masked row); the others see keys 0 .. i - (sq - sk)."""
+    lens_q, lens_k = [48, 70, 40], [16, 64, 40]
+    q, k, v, cu_q, cu_k = _packed_case(gpu, lens_q, lens_k, 16, 8, seed=13)
+    out = ops.flash_attn_varlen_func(q, k, v, max_seqlen_q=max(lens_q), cu_seqlens_q=cu_q, max_seqlen_k=max(lens_k),
+                                     cu_seqlens_k=cu_k, causal=True)
+    torch.cuda.synchronize()
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    aq = ak = 0
+    for nq, nk in zip(lens_q, lens_k):
+        dead = max(nq - nk, 0)
+        assert (got[aq:aq + dead] == 0).all()
+        live = nq - dead                                    # the last `live` queries against the first nk keys, sq == sk form
+        qq = q[aq + dead:aq + nq].float().cpu().permute(1, 0, 2)
+        kk = k[ak:ak + nk].float().cpu().permute(1, 0, 2).repeat_interleave(2, 0)
+        vv = v[ak:ak + nk].float().cpu().permute(1, 0, 2).repeat_interleave(2, 0)
+        mask = torch.ones(live, nk, dtype=torch.bool).tril(diagonal=nk - live)
+        ref = torch.nn.functional.scaled_dot_product_attention(qq, kk, vv, attn_mask=mask).permute(1, 0, 2)
+        assert (got[aq + dead:aq + nq] - ref).abs().max() <= ATTN_ATOL
+        aq += nq
+        ak += nk
+
+
 @pytest.mark.parametrize("scale", [0.02, 0.25])
 def test_softmax_scale_is_honoured(gpu, scale):
     wl = workloads.make_prefill_workload("p", [90, 300, 700], [0, 256, 512], 32, 8, seed=21, pad_fraction=0.0).to(gpu)
