@@ -124,6 +124,27 @@ def test_row_maximum_covers_every_key_of_a_step(gpu):
         assert np.array_equal(got[i, ::g], f32(wl.v_cache[blk, pos % wl.block_size]))
 
 
+@pytest.mark.parametrize("direction", [1, -1])
+def test_scores_that_rise_or_fall_along_the_sequence(gpu, direction):
+    """Keys that are multiples of the query, the factor rising (or falling) by a fixed amount per token: the
+    running maximum grows at every step (the accumulators are rescaled every time), or is set by the very
+    first key and never again, with all later keys hundreds of log2 units below it."""
+    lens = [700, 257, 33, 1024]
+    wl = workloads.make_decode_workload("ramp", lens, 16, 8, seed=13).to(gpu)
+    g = wl.num_q_heads // wl.num_kv_heads
+    for i, n in enumerate(lens):
+        q0 = wl.q[i, ::g].float()                                         # [Hkv, D]
+        unit = q0 / (wl.scale * (q0 * q0).sum(dim=-1, keepdim=True))      # score * scale = 1 per unit factor
+        for pos in range(n):
+            f = 0.5 * (pos if direction > 0 else -pos)                   # 16 log2-ish units per 32-token step
+            blk = int(wl.block_table[i, pos // wl.block_size])
+            wl.k_cache[blk, pos % wl.block_size] = (f * unit).to(torch.bfloat16)
+    got = f32(gpu_decode(wl))
+    want = oracle_decode(wl)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= ATTN_ATOL
+
+
 def test_block_permutation_invariance(gpu):
     """Same logical tokens under a different physical placement give bit-identical output."""
     wl = workloads.make_decode_workload("perm", [700, 1023, 40], 32, 8, nblk=32, seed=7).to(gpu)

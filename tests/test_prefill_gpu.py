@@ -69,6 +69,35 @@ def test_row_maximum_covers_every_key_of_a_step(gpu):
         assert np.array_equal(got[p:96 * (j + 1), ::g], np.broadcast_to(f32(wl.v_new[p]), (96 * (j + 1) - p, 8, 128)))
 
 
+@pytest.mark.parametrize("direction", [1, -1])
+def test_scores_that_rise_or_fall_along_the_sequence(gpu, direction):
+    """Keys that are multiples of one query vector shared by a prompt, the factor rising (or falling) by a
+    fixed amount per token: the running maximum of every query row grows at every step, or is set by key 0
+    and never again, with the later keys hundreds of log2 units below it."""
+    lens = [300, 97, 640]
+    wl = workloads.make_prefill_workload("ramp", lens, [0, 0, 256], 16, 8, seed=14, pad_fraction=0.0).to(gpu)
+    g = wl.num_q_heads // wl.num_kv_heads
+    kc, vc = wl.k_cache.clone(), wl.v_cache.clone()
+    ops.store_kvcache(wl.k_new, wl.v_new, kc, vc, wl.slot_mapping)
+    aq = 0
+    for i, (n, c) in enumerate(zip(lens, wl.cached)):
+        wl.q[aq:aq + n - c] = wl.q[aq]
+        q0 = wl.q[aq, ::g].float()
+        unit = q0 / (wl.scale * (q0 * q0).sum(dim=-1, keepdim=True))
+        for pos in range(n):
+            f = 0.5 * (pos if direction > 0 else -pos)
+            blk = int(wl.block_table[i, pos // wl.block_size])
+            kc[blk, pos % wl.block_size] = (f * unit).to(torch.bfloat16)
+        aq += n - c
+    out = ops.flash_attn_varlen_func(wl.q, kc, vc, max_seqlen_q=wl.max_seqlen_q, cu_seqlens_q=wl.cu_seqlens_q,
+                                     max_seqlen_k=wl.max_seqlen_k, cu_seqlens_k=wl.cu_seqlens_k,
+                                     softmax_scale=wl.scale, causal=True, block_table=wl.block_table)
+    torch.cuda.synchronize()
+    got, want = f32(out), oracle_paged(wl, kc, vc)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= ATTN_ATOL
+
+
 @pytest.mark.parametrize("bs", [32, 64, 512])
 def test_block_sizes(gpu, bs):
     wl = workloads.make_prefill_workload("p", [70, 200, 5], [bs if bs <= 64 else 0, 0, 0], 16, 8, bs=bs, seed=bs,
