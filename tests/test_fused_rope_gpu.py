@@ -66,6 +66,37 @@ def test_against_oracle(gpu, n, hq, hkv):
     assert np.array_equal(bits(kc).reshape(-1, width)[untouched], ek.reshape(-1, width)[untouched])
 
 
+def test_rows_of_extreme_magnitude(gpu):
+    """Head rows of zeros (variance 0: the norm is eps alone), of very large, very small and alternating
+    magnitudes: the sums of squares and the products keep float32 range and the reference's rounding points."""
+    n, hq, hkv = 48, 32, 8
+    qkv, q, k, v, wq, wk, cache, pos, kc, vc, slots = make(n, hq, hkv, 77, gpu)
+    with torch.no_grad():
+        q[0::6] = 0
+        k[0::6] = 0
+        q[1::6] *= 1000.0
+        k[1::6] *= 1000.0
+        q[2::6] *= 1e-3
+        k[2::6] *= 1e-3
+        q[3::6, :, ::2] *= 300.0                                   # large and small elements side by side
+        k[3::6, :, 1::2] *= 1e-2
+    ek, ev = bits(kc).copy(), bits(vc).copy()
+    q2, k2 = R.qk_norm_rope_append_ref(bits(q.contiguous()), bits(k.contiguous()), bits(v.contiguous()),
+                                       pos.cpu().numpy(), bits(wq), bits(wk), 1e-6, bits(cache), ek, ev,
+                                       slots.cpu().numpy())
+    ops.qk_norm_rope_store_kvcache(q, k, v, pos, wq, wk, 1e-6, cache, kc, vc, slots)
+    torch.cuda.synchronize()
+    keep = np.arange(n) % 6 != 0                                   # the zero rows are compared as values: +0 and -0 are both right
+    gq, gk = bits(q.contiguous()), bits(k.contiguous())
+    close(gq[keep], q2[keep])
+    close(gk[keep], k2[keep])
+    assert np.array_equal(bits(vc), ev)
+    assert (gq[~keep] & 0x7fff == 0).all() and (q2[~keep] & 0x7fff == 0).all()
+    assert (gk[~keep] & 0x7fff == 0).all() and (k2[~keep] & 0x7fff == 0).all()
+    got_kc, want_kc = bf16_to_f32(bits(kc)), bf16_to_f32(ek)
+    assert np.abs(got_kc - want_kc).max() <= 1e-2 + 1e-2 * np.abs(want_kc).max()
+
+
 def test_key_can_be_left_untouched(gpu):
     qkv, q, k, v, wq, wk, cache, pos, kc, vc, slots = make(20, 16, 8, 3, gpu, pad_every=0)
     k_before = k.clone()
