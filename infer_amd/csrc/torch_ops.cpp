@@ -31,11 +31,13 @@ void check_bf16_cuda(const at::Tensor& t, const char* name) {
 // stays alive for the life of the process: a HIP graph captured at the smaller batch still points
 // at it, and its replays must keep writing to memory nobody else owns.  The buffer is shared by all
 // calls for the shape, so those calls must be ordered on one stream (the partial results of one call
-// are live until its merge kernel has run); callers that decode the same shape on several streams
-// at once call infer_paged_decode_bf16 with a workspace per stream instead.
+// are live until its merge kernel has run): a call that arrives on another stream while the last one is
+// still busy is refused; callers that decode the same shape on several streams at once call
+// infer_paged_decode_bf16 with a workspace per stream instead.
 at::Tensor decode_workspace(const at::Tensor& like, int64_t batch, int64_t hq, int64_t hkv, int64_t d) {
     static std::mutex mu;
     static std::unordered_map<std::string, std::pair<int64_t, at::Tensor>> cache;
+    static std::unordered_map<std::string, hipStream_t> last_stream;
     static std::vector<at::Tensor> retired;
     std::lock_guard<std::mutex> g(mu);
     const std::string key = std::to_string(like.get_device()) + ":" + std::to_string(hq) + ":" + std::to_string(hkv) + ":" + std::to_string(d);
@@ -47,6 +49,19 @@ at::Tensor decode_workspace(const at::Tensor& like, int64_t batch, int64_t hq, i
         if (slot.second.defined()) retired.push_back(slot.second);
         slot = {cap, at::empty({static_cast<int64_t>(bytes)}, like.options().dtype(at::kByte))};
     }
+    // a call on another stream while the last one still has work pending would overwrite partial results
+    // in use: refused (checked on a change of stream only; streams under capture are not queried)
+    const hipStream_t cur = static_cast<hipStream_t>(current_stream());
+    auto it = last_stream.find(key);
+    if (it != last_stream.end() && it->second != cur) {
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        const bool capturing = hipStreamIsCapturing(cur, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone;
+        const bool busy = !capturing && hipStreamQuery(it->second) == hipErrorNotReady;
+        (void)hipGetLastError();
+        TORCH_CHECK(!busy, "paged decode: the shared workspace is still in use on another stream; order the calls on one "
+                           "stream, or call infer_paged_decode_bf16 with a workspace per stream");
+    }
+    last_stream[key] = cur;
     return slot.second;
 }
 

@@ -127,6 +127,22 @@ def decode_workspace(device, max_batch: int, num_q_heads: int, num_kv_heads: int
     return ws[1]
 
 
+_workspace_streams: dict = {}      # data_ptr of a shared workspace -> the stream that used it last
+
+
+def _claim_shared_workspace(workspace: torch.Tensor, device) -> None:
+    """The shared workspace holds the partial results of a call until its merge kernel has run, so calls
+    that use it must be ordered on one stream.  A call on another stream while the last one still has work
+    pending is refused (a host-side check on a change of stream only; streams under capture are not
+    queried): pass ``workspace=`` of its own to such a call."""
+    cur = torch.cuda.current_stream(device)
+    last = _workspace_streams.get(workspace.data_ptr())
+    if last is not None and last != cur and not torch.cuda.is_current_stream_capturing() and not last.query():
+        raise RuntimeError("paged decode: the shared workspace is still in use on another stream; "
+                           "order the calls on one stream or pass a workspace of their own")
+    _workspace_streams[workspace.data_ptr()] = cur
+
+
 def _decode_args(q3, k_cache, v_cache, cache_seqlens, block_table):
     assert q3.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16
     uniform = isinstance(cache_seqlens, int)      # one length for the whole batch, known on the host
@@ -160,6 +176,7 @@ def paged_attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     assert out.shape == q.shape and out.dtype == torch.bfloat16 and out.stride(2) == 1 and out.stride(1) == d
     if workspace is None:
         workspace = decode_workspace(q.device, b, hq, hkv, d)
+        _claim_shared_workspace(workspace, q.device)
     lib = _lib.load()
     if isinstance(context_lens, int):
         rc = lib.infer_paged_decode_uniform_bf16(

@@ -351,6 +351,28 @@ def test_two_streams_with_different_split_counts(gpu):
         assert float(np.abs(f32(got) - oracle_decode(wl)).max()) <= ATTN_ATOL
 
 
+def test_shared_workspace_refuses_a_second_stream_while_the_first_is_busy(gpu):
+    """Calls without a workspace of their own share one per shape, which holds partial results until the
+    merge kernel has run: a call on another stream while the last stream still has work pending is refused
+    instead of overwriting them; once that stream is idle the other one may use it."""
+    wl = workloads.make_decode_workload("ws", [900, 300, 2000, 64], 32, 8, seed=21).to(gpu)
+    out = torch.empty_like(wl.q)
+    call = lambda: ops.paged_attn_decode(wl.q, wl.k_cache, wl.v_cache, wl.block_table, wl.context_lens, wl.scale, out)
+    torch.cuda.synchronize()
+    sa, sb = torch.cuda.Stream(), torch.cuda.Stream()
+    with torch.cuda.stream(sa):
+        torch.cuda._sleep(200_000_000)          # keeps stream sa busy for a moment
+        call()
+    with torch.cuda.stream(sb):
+        with pytest.raises(RuntimeError, match="still in use on another stream"):
+            call()
+    sa.synchronize()
+    with torch.cuda.stream(sb):
+        call()
+    torch.cuda.synchronize()
+    assert float(np.abs(f32(out) - oracle_decode(wl)).max()) <= ATTN_ATOL
+
+
 def test_split_then_merge_need_not_agree_on_a_setting(gpu):
     """The merge phase locates the partial results from the workspace alone: a split launched with any
     split count is merged correctly by the same merge call."""

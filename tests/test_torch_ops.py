@@ -48,6 +48,30 @@ def test_torch_ops_match_the_oracle(gpu):
 
 
 @pytest.mark.gpu
+def test_torch_op_workspace_refuses_a_second_stream_while_the_first_is_busy(gpu):
+    """torch.ops._C.paged_attn_decode keeps one workspace per shape: a call on another stream while the last
+    stream still has work pending raises instead of overwriting partial results in use."""
+    import infer_ops
+    wl = workloads.make_decode_workload("tws", [700, 90, 1500, 33, 260], 16, 8, seed=22).to(gpu)
+    out = torch.empty_like(wl.q)
+    call = lambda: infer_ops.paged_attn_decode(wl.q, wl.k_cache, wl.v_cache, wl.block_table, wl.context_lens,
+                                               wl.scale, out)
+    torch.cuda.synchronize()
+    sa, sb = torch.cuda.Stream(), torch.cuda.Stream()
+    with torch.cuda.stream(sa):
+        torch.cuda._sleep(200_000_000)
+        call()
+    with torch.cuda.stream(sb):
+        with pytest.raises(RuntimeError, match="still in use on another stream"):
+            call()
+    sa.synchronize()
+    with torch.cuda.stream(sb):
+        call()
+    torch.cuda.synchronize()
+    assert np.abs(f32(out) - oracle_decode(wl)).max() <= ATTN_ATOL
+
+
+@pytest.mark.gpu
 def test_registry_operators_run_the_kernels(gpu):
     """KVAppendOperator / PagedAttentionOperator are fetched from the OperatorRegistry through the
     UnifiedOp facade and really override forward()."""
