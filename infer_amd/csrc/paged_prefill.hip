@@ -221,11 +221,11 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
     for (int i = 0; i < 8; ++i) ones[i] = (__bf16)1.0f;
 #pragma unroll
     for (int u = 0; u < kNQ; ++u) {
-        const u32x4 z = {0u, 0u, 0u, 0u};
-        const bool live = my_q[u] < sq;
-        const uint16_t* qp = a.q + (int64_t)(q_beg + (live ? my_q[u] : 0)) * a.q_stride0 + (int64_t)head * kD + 8 * g;
+        // lanes behind the last query of the sequence load its first query instead: straight-line loads,
+        // finite values, and their columns of the result are never stored
+        const uint16_t* qp = a.q + (int64_t)(q_beg + (my_q[u] < sq ? my_q[u] : 0)) * a.q_stride0 + (int64_t)head * kD + 8 * g;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) qreg[u][j] = as_bf16x8(live ? load16(qp + 32 * j) : z);
+        for (int j = 0; j < 4; ++j) qreg[u][j] = as_bf16x8(load16(qp + 32 * j));
     }
     f32x4 acc[kNQ][8];
     // Row sums ride the matrix pipe: ones[16 x 32] . P^T adds the 32 probabilities of a step for every
