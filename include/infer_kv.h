@@ -246,7 +246,8 @@ int infer_paged_decode_noalloc_bf16(const void* q, int64_t q_stride0,
  * kv_rows = number of token rows addressable through k/v (packed: rows of the tensor; paged:
  * num_blocks * block_size); it only bounds reads.  causal != 0 applies the bottom-right aligned
  * mask (key j visible to query i of the sequence iff j <= i + (sk - sq)).  Queries of a sequence
- * with sk == 0 produce zeros.  With a block table, table_cols is the number of entries per row
+ * with sk == 0 produce zeros, and so do the first sq - sk queries of a sequence with sq > sk (no key is
+ * visible to them).  With a block table, table_cols is the number of entries per row
  * (bt_stride0 >= table_cols) and a key length beyond table_cols * block_size is cut to that.  scale
  * must be positive (INFER_KV_EINVAL otherwise).  Same shape limits as the decode entry points.  No
  * workspace.
